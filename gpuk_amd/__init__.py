@@ -1,0 +1,129 @@
+"""gpuk_amd -- MI355X (gfx950) implementation of gpuk's memory-bound fused inference ops.
+
+Mirrors the reference's Python shim (gpuk/__init__.py): importing the package loads the torch
+library `gpuk` and binds the operator names as module attributes, so
+
+    import gpuk_amd as gpuk
+    gpuk.fused_rope_rms(qkv, qw, kw, cos_sin, positions, T, Hq, Hk, Hv, D, True, 1e-6)
+    env = gpuk.GPUKDistEnv(device_id=0); env.allreduce_add_rms_fused(x, residual, gamma, eps, fp8_out=True)
+
+works as with the reference (gpuk/__init__.py:18-35, :54-205).  Only the operators of the two fused
+paths exist here; there is no CPU or pure-torch fallback: if the built libraries are missing the
+import raises.
+"""
+from __future__ import annotations
+
+import os
+from contextlib import contextmanager
+from typing import Optional
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_PKG_DIR, "lib")
+KERNEL_LIB = os.path.join(LIB_DIR, "libgpuk_amd.so")   # C ABI, include/gpuk_amd.h
+TORCH_LIB = os.path.join(LIB_DIR, "libgpuk.so")        # TORCH_LIBRARY(gpuk, ...)
+
+if not (os.path.exists(KERNEL_LIB) and os.path.exists(TORCH_LIB)):
+    raise ImportError(
+        f"gpuk_amd: {KERNEL_LIB} / {TORCH_LIB} not built; run `python -m gpuk_amd.build` "
+        "(hipcc cross-compiles gfx950 without a GPU). There is no fallback path.")
+
+torch.ops.load_library(TORCH_LIB)
+
+allreduce_rms = torch.ops.gpuk.allreduce_rms
+fused_rope_rms = torch.ops.gpuk.fused_rope_rms
+fused_mrope_3d_rms = torch.ops.gpuk.fused_mrope_3d_rms
+fused_mrope_3d_rms_set_kv = torch.ops.gpuk.fused_mrope_3d_rms_set_kv
+fused_rope_rms_set_kv = torch.ops.gpuk.fused_rope_rms_set_kv       # additive: 1-D positions + KV write
+set_fp8_max = torch.ops.gpuk.set_fp8_max                           # additive
+get_fp8_max = torch.ops.gpuk.get_fp8_max                           # additive
+
+# gfx950 encodes OCP e4m3fn.  The reference defaults to the MI300-only e4m3fnuz (gpuk/__init__.py:38)
+# and uses 240 as e4m3fn's maximum (:42-46); 448 is the OCP maximum.  `set_fp8_max(240)` restores the
+# reference's divisor (codes up to 240 are identical in both encodings).
+fp8 = torch.float8_e4m3fn
+fp8_max_val_ = {torch.float8_e4m3fn: 448}
+fp8_max_val = fp8_max_val_[fp8]
+fp8_policy_id_ = {torch.float8_e4m3fn: 1}
+fp8_policy_id = fp8_policy_id_[fp8]
+
+QUANT_NONE = 0
+QUANT_FP8_DYNAMIC = 1
+QUANT_FP8_STATIC = 3   # additive: one per-tensor scale, read from scale_out[0]
+
+
+class GPUKDistEnv:
+    """Single-GPU counterpart of the reference's GPUKDistEnv (gpuk/__init__.py:54-205).
+
+    The reference returns early with `fptr = None` at world size 1 and cannot run the fused op there
+    (:72-73); here world size 1 is the supported case: `fptr` is 0 and `allreduce_add_rms_fused` runs
+    residual-add + RMSNorm + quant with `allreduce_in` taken as the already-reduced activation.
+    A larger world size raises: the IPC workspace and the all-reduce kernels are not part of this build.
+    """
+
+    _SUPPORTED_WORLD_SIZES = [1]
+
+    def __init__(self, group=None, device_id: Optional[int] = None, max_size_in_bytes=16384 * 16384,
+                 comm_ptrs_buf_len=1024 * 256, dtype: torch.dtype = torch.bfloat16) -> None:
+        import torch.distributed as dist
+
+        self.group = group
+        self.device_id = device_id if device_id is not None else torch.cuda.current_device()
+        if dist.is_available() and dist.is_initialized():
+            self.rank = dist.get_rank(group=self.group)
+            self.world_size = dist.get_world_size(group=self.group)
+        else:
+            self.rank, self.world_size = 0, 1
+        if self.world_size not in GPUKDistEnv._SUPPORTED_WORLD_SIZES:
+            raise NotImplementedError(
+                f"GPUKDistEnv: world size {self.world_size} needs the cross-GPU all-reduce workspace, "
+                "which this single-GPU build does not contain")
+        self.fptr = 0
+        self.disabled = False
+        self._IS_CAPTURING = False
+        self._IS_CAPTURED = False
+        torch.cuda.set_device(self.device_id)
+
+    def barrier(self):
+        torch.cuda.set_device(self.device_id)
+        torch.cuda.synchronize(self.device_id)
+
+    def consume_capture(self):
+        """No peer pointers to exchange at world size 1 (reference: gpuk/__init__.py:98-110)."""
+        self.barrier()
+
+    @contextmanager
+    def capture(self):
+        try:
+            self._IS_CAPTURING = True
+            yield
+        finally:
+            self._IS_CAPTURING = False
+
+    def allreduce_native(self, allreduce_in):
+        return allreduce_in.clone()
+
+    def allreduce(self, allreduce_in):
+        return allreduce_in.clone()
+
+    def allreduce_add_rms_fused(self, allreduce_in, residual_in, rms_weight, eps, fp8_out=False, static_scale=None):
+        """gpuk/__init__.py:175-205.  Returns (residual_out, norm_out, scale_out).
+
+        `static_scale` (additive): a 1-element fp32 tensor; selects per-tensor static quantisation.
+        """
+        residual_out = torch.empty_like(residual_in)
+        if fp8_out:
+            norm_out = torch.empty_like(allreduce_in, dtype=fp8)
+            if static_scale is not None:
+                scale_out = static_scale.reshape(1).to(device=allreduce_in.device, dtype=torch.float32).contiguous()
+                quant = QUANT_FP8_STATIC
+            else:
+                scale_out = torch.empty(allreduce_in.shape[0], 1, dtype=torch.float32, device=allreduce_in.device)
+                quant = fp8_policy_id
+        else:
+            norm_out = torch.empty_like(allreduce_in)
+            scale_out = torch.empty(1, dtype=torch.float32, device=allreduce_in.device)
+            quant = QUANT_NONE
+        allreduce_rms(self.fptr, allreduce_in, residual_in, rms_weight, residual_out, norm_out, scale_out, eps, quant)
+        return residual_out, norm_out, scale_out

@@ -1,0 +1,114 @@
+"""ctypes binding of the C ABI (include/gpuk_amd.h) for callers that hold raw device pointers.
+
+Takes torch tensors only to read `data_ptr()`; the launches go on torch's current stream unless a
+stream handle is given.  Raises GpukError on a non-zero status.  No fallback of any kind.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional, Sequence
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libgpuk_amd.so")
+
+EXPORTS = ("gpuk_status_string", "gpuk_abi_version", "gpuk_add_rmsnorm_quant", "gpuk_rope_rms",
+           "gpuk_rope_rms_set_kv", "gpuk_set_tuning")
+
+DTYPE = {torch.bfloat16: 0, torch.float16: 1}
+QUANT_NONE, QUANT_FP8_DYNAMIC, QUANT_FP8_E4M3FNUZ, QUANT_FP8_STATIC = 0, 1, 2, 3
+KV_SAME, KV_E4M3FN = 0, 1
+
+
+class GpukError(RuntimeError):
+    def __init__(self, status: int, what: str):
+        self.status = status
+        super().__init__(f"{what}: {lib().gpuk_status_string(status).decode()} (status {status})")
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise ImportError(f"{_LIB_PATH} not built; run `python -m gpuk_amd.build`")
+        L = C.CDLL(_LIB_PATH)
+        L.gpuk_status_string.restype = C.c_char_p
+        L.gpuk_status_string.argtypes = [C.c_int]
+        L.gpuk_abi_version.restype = C.c_int
+        L.gpuk_set_tuning.restype = C.c_int
+        L.gpuk_set_tuning.argtypes = [C.c_char_p, C.c_int]
+        L.gpuk_add_rmsnorm_quant.restype = C.c_int
+        L.gpuk_add_rmsnorm_quant.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int64, C.c_float, C.c_int, C.c_int,
+                                                               C.c_float, C.c_void_p]
+        rope_head = [C.c_void_p] * 5 + [C.c_int64, C.c_int64, C.c_int] + [C.c_int64] * 5 + [
+            C.c_int, C.POINTER(C.c_int64), C.c_int, C.c_float, C.c_int]
+        L.gpuk_rope_rms.restype = C.c_int
+        L.gpuk_rope_rms.argtypes = rope_head + [C.c_void_p]
+        L.gpuk_rope_rms_set_kv.restype = C.c_int
+        L.gpuk_rope_rms_set_kv.argtypes = rope_head + [C.c_void_p] * 4 + [C.c_float, C.c_float, C.c_int, C.c_void_p]
+        _lib = L
+    return _lib
+
+
+def _stream(stream) -> int:
+    if stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    return getattr(stream, "cuda_stream", stream)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def set_tuning(key: str, value: int) -> None:
+    rc = lib().gpuk_set_tuning(key.encode(), value)
+    if rc:
+        raise GpukError(rc, f"gpuk_set_tuning({key})")
+
+
+def add_rmsnorm_quant(x, residual_in, gamma, residual_out, norm_out, scale, eps: float, quant: int,
+                      fp8_max: float = 448.0, stream=None) -> None:
+    tokens = x.numel() // x.shape[-1] if x.shape[-1] else 0
+    rc = lib().gpuk_add_rmsnorm_quant(_ptr(x), _ptr(residual_in), _ptr(gamma), _ptr(residual_out), _ptr(norm_out),
+                                      _ptr(scale), tokens, x.shape[-1], eps, DTYPE[x.dtype], quant, fp8_max,
+                                      _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_add_rmsnorm_quant")
+
+
+def _pos_args(positions):
+    if positions.dim() == 1:
+        return 0, positions.stride(0), 1
+    return positions.stride(0), positions.stride(1), 3
+
+
+def _section(mrope_section: Optional[Sequence[int]]):
+    if mrope_section is None:
+        return None
+    return (C.c_int64 * 3)(*[int(v) for v in mrope_section])
+
+
+def rope_rms(qkv, qw, kw, cos_sin, positions, T, Hq, Hk, Hv, D, is_neox, eps, mrope_section=None,
+             is_interleaved=False, stream=None) -> None:
+    psa, pst, n_axes = _pos_args(positions)
+    rc = lib().gpuk_rope_rms(_ptr(qkv), _ptr(qw), _ptr(kw), _ptr(cos_sin), _ptr(positions), psa, pst, n_axes,
+                             T, Hq, Hk, Hv, D, int(is_neox), _section(mrope_section), int(is_interleaved), eps,
+                             DTYPE[qkv.dtype], _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_rope_rms")
+
+
+def rope_rms_set_kv(qkv, qw, kw, cos_sin, positions, T, Hq, Hk, Hv, D, is_neox, eps, q_out, k_cache, v_cache, kv_loc,
+                    k_scale=1.0, v_scale=1.0, mrope_section=None, is_interleaved=False, stream=None) -> None:
+    psa, pst, n_axes = _pos_args(positions)
+    kv = KV_SAME if k_cache.dtype == qkv.dtype else KV_E4M3FN
+    rc = lib().gpuk_rope_rms_set_kv(_ptr(qkv), _ptr(qw), _ptr(kw), _ptr(cos_sin), _ptr(positions), psa, pst, n_axes,
+                                    T, Hq, Hk, Hv, D, int(is_neox), _section(mrope_section), int(is_interleaved), eps,
+                                    DTYPE[qkv.dtype], _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _ptr(kv_loc),
+                                    k_scale, v_scale, kv, _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_rope_rms_set_kv")

@@ -1,0 +1,337 @@
+// residual-add -> RMSNorm -> (optional) FP8 e4m3fn quantisation, one workgroup per token row.
+//
+// This is the one-GPU share of the reference's all-reduce-fusion epilogue: the residual add at
+// src/impl/all_reduce_fusion_impl.h:256-265 followed by epilogue<>() at :202-228 (rms_norm :159-181,
+// reduce_abs_max :183-200, convert_to_fp8 :148-157), reached through the allreduce_rms host op
+// (src/ops/all_reduce_fusion.cpp:363-396).  There is no all-reduce here.
+//
+// Numerics follow the reference's torch oracle (gpuk/__init__.py:147-164) op by op, *not* the
+// reference kernel (which keeps fp32 until the fp8 cast):
+//     res  = rT(x + r)                       rT = round-to-nearest-even into the 16-bit type
+//     var  = sum(res^2) / H ; rstd = 1 / sqrt(var + eps)          (correctly rounded sqrt and divide)
+//     n1   = rT(res * rstd) ; n2 = rT(gamma * n1)
+//     scale = amax|n2| / fp8_max  (1 when the row is all zero, as the reference kernel: :217)
+//     code = e4m3fn_rne(clamp(n2 / scale, +-fp8_max))             (fp32 IEEE quotient)
+//
+// Data movement per element: 2 B x + 2 B residual in, 2 B residual out, 1 B code (7 B); the row lives
+// in registers between the three phases, so HBM sees each byte once.  Lane `t` of the workgroup owns
+// 16-byte chunk `i*blockDim + t` of the row for i < NCHUNK: every wave load/store instruction covers
+// 1 KiB (loads) or 512 B (codes) of contiguous memory.
+#include <hip/hip_runtime.h>
+
+#include "../../../include/gpuk_amd.h"
+#include "device_utils.h"
+#include "host_utils.h"
+
+namespace gpuk {
+
+namespace {
+
+constexpr int kMaxThreads = 1024;
+constexpr int kMaxWaves = kMaxThreads / 64;
+
+template <typename V>
+__device__ __forceinline__ V load_stream(const V *p) { return __builtin_nontemporal_load(p); }
+template <typename V>
+__device__ __forceinline__ void store_stream(V *p, V v) { __builtin_nontemporal_store(v, p); }
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// The scale reciprocal is usable by div_by_rcp when scale is comfortably normal.
+__device__ __forceinline__ bool scale_in_fast_range(float s) {
+    return s >= 0x1p-60f && s <= 0x1p60f;
+}
+
+template <typename T, int NCHUNK, int QUANT>
+__global__ void __launch_bounds__(kMaxThreads)
+add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ residual_in,
+                       const u32x4 *__restrict__ gamma, u32x4 *__restrict__ residual_out,
+                       void *__restrict__ norm_out, float *__restrict__ scale_io, int chunks_per_row,
+                       float hidden_f, float eps, float fp8_max) {
+    using P = Pack16<T>;
+    __shared__ float s_sum[kMaxWaves];
+    __shared__ float s_max[kMaxWaves];
+
+    const int tid = threadIdx.x;
+    const int num_waves = blockDim.x >> 6;
+    const int64_t row_base = (int64_t)blockIdx.x * chunks_per_row;
+
+    // ---- phase 0: issue every load of the row before touching any of them
+    u32x4 xv[NCHUNK], rv[NCHUNK], gv[NCHUNK];
+    bool live[NCHUNK];
+#pragma unroll
+    for (int i = 0; i < NCHUNK; ++i) {
+        const int c = i * blockDim.x + tid;
+        live[i] = c < chunks_per_row;
+        if (live[i]) {
+            xv[i] = load_stream(x + row_base + c);
+            rv[i] = load_stream(residual_in + row_base + c);
+        } else {
+            xv[i] = u32x4{0, 0, 0, 0};
+            rv[i] = u32x4{0, 0, 0, 0};
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NCHUNK; ++i) {
+        const int c = i * blockDim.x + tid;
+        gv[i] = live[i] ? gamma[c] : u32x4{0, 0, 0, 0};
+    }
+
+    // ---- phase 1: res = rT(x + r), stored once; sum of squares of the *rounded* residual
+    float ss0 = 0.f, ss1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCHUNK; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t w = P::pack(P::lo(xv[i][j]) + P::lo(rv[i][j]), P::hi(xv[i][j]) + P::hi(rv[i][j]));
+            xv[i][j] = w;  // xv now holds the residual
+            const float a = P::lo(w), b = P::hi(w);
+            ss0 = __builtin_fmaf(a, a, ss0);
+            ss1 = __builtin_fmaf(b, b, ss1);
+        }
+        if (live[i]) store_stream(residual_out + row_base + i * blockDim.x + tid, xv[i]);
+    }
+    const float sumsq = block_allreduce<SumOp>(ss0 + ss1, s_sum, num_waves);
+    const float rstd = 1.0f / sqrtf(sumsq / hidden_f + eps);
+
+    // ---- phase 2: n2 = rT(gamma * rT(res * rstd)); row amax for the dynamic scale
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCHUNK; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t n1 = P::pack(P::lo(xv[i][j]) * rstd, P::hi(xv[i][j]) * rstd);
+            const uint32_t n2 = P::pack(P::lo(gv[i][j]) * P::lo(n1), P::hi(gv[i][j]) * P::hi(n1));
+            xv[i][j] = n2;  // xv now holds the normed row
+            if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
+                amax = __builtin_fmaxf(amax, __builtin_fabsf(P::lo(n2)));
+                amax = __builtin_fmaxf(amax, __builtin_fabsf(P::hi(n2)));
+            }
+        }
+    }
+
+    if constexpr (QUANT == GPUK_QUANT_NONE) {
+        u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base;
+#pragma unroll
+        for (int i = 0; i < NCHUNK; ++i)
+            if (live[i]) store_stream(out + i * blockDim.x + tid, xv[i]);
+        return;
+    } else {
+        float scale;
+        if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
+            amax = block_allreduce<MaxOp>(amax, s_max, num_waves);
+            scale = amax == 0.f ? 1.f : amax / fp8_max;
+            if (tid == 0) scale_io[blockIdx.x] = scale;
+        } else {
+            scale = scale_io[0];
+        }
+
+        // ---- phase 3: code = e4m3fn(clamp(n2 / scale)); 8 codes (one 8-byte store) per chunk
+        u32x2 *out = reinterpret_cast<u32x2 *>(norm_out) + row_base;
+        if (scale_in_fast_range(scale)) {
+            const float rcp = 1.0f / scale;
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i) {
+                float q[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    q[2 * j] = clamp_sym(div_by_rcp(P::lo(xv[i][j]), scale, rcp), fp8_max);
+                    q[2 * j + 1] = clamp_sym(div_by_rcp(P::hi(xv[i][j]), scale, rcp), fp8_max);
+                }
+                u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                if (live[i]) store_stream(out + i * blockDim.x + tid, codes);
+            }
+        } else {
+#pragma unroll 1
+            for (int i = 0; i < NCHUNK; ++i) {
+                float q[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    q[2 * j] = clamp_sym(P::lo(xv[i][j]) / scale, fp8_max);
+                    q[2 * j + 1] = clamp_sym(P::hi(xv[i][j]) / scale, fp8_max);
+                }
+                u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                if (live[i]) store_stream(out + i * blockDim.x + tid, codes);
+            }
+        }
+    }
+}
+
+// Rows too long to keep in registers (more than 8 chunks per lane at 1024 lanes, i.e. hidden > 65536):
+// three sweeps over the row, re-reading what this same lane wrote to residual_out (L2-resident).
+template <typename T, int QUANT>
+__global__ void __launch_bounds__(kMaxThreads)
+add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ residual_in,
+                            const u32x4 *__restrict__ gamma, u32x4 *residual_out, void *__restrict__ norm_out,
+                            float *__restrict__ scale_io, int chunks_per_row, float hidden_f, float eps,
+                            float fp8_max) {
+    using P = Pack16<T>;
+    __shared__ float s_sum[kMaxWaves];
+    __shared__ float s_max[kMaxWaves];
+    const int tid = threadIdx.x;
+    const int num_waves = blockDim.x >> 6;
+    const int64_t row_base = (int64_t)blockIdx.x * chunks_per_row;
+
+    float ss = 0.f;
+    for (int c = tid; c < chunks_per_row; c += blockDim.x) {
+        u32x4 xv = x[row_base + c], rv = residual_in[row_base + c];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t w = P::pack(P::lo(xv[j]) + P::lo(rv[j]), P::hi(xv[j]) + P::hi(rv[j]));
+            xv[j] = w;
+            ss = __builtin_fmaf(P::lo(w), P::lo(w), ss);
+            ss = __builtin_fmaf(P::hi(w), P::hi(w), ss);
+        }
+        residual_out[row_base + c] = xv;
+    }
+    const float sumsq = block_allreduce<SumOp>(ss, s_sum, num_waves);
+    const float rstd = 1.0f / sqrtf(sumsq / hidden_f + eps);
+
+    auto normed = [&](int c) {
+        u32x4 v = residual_out[row_base + c];  // written by this lane above
+        const u32x4 g = gamma[c];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t n1 = P::pack(P::lo(v[j]) * rstd, P::hi(v[j]) * rstd);
+            v[j] = P::pack(P::lo(g[j]) * P::lo(n1), P::hi(g[j]) * P::hi(n1));
+        }
+        return v;
+    };
+
+    if constexpr (QUANT == GPUK_QUANT_NONE) {
+        u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base;
+        for (int c = tid; c < chunks_per_row; c += blockDim.x) out[c] = normed(c);
+    } else {
+        float scale;
+        if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
+            float amax = 0.f;
+            for (int c = tid; c < chunks_per_row; c += blockDim.x) {
+                const u32x4 v = normed(c);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    amax = __builtin_fmaxf(amax, __builtin_fabsf(P::lo(v[j])));
+                    amax = __builtin_fmaxf(amax, __builtin_fabsf(P::hi(v[j])));
+                }
+            }
+            amax = block_allreduce<MaxOp>(amax, s_max, num_waves);
+            scale = amax == 0.f ? 1.f : amax / fp8_max;
+            if (tid == 0) scale_io[blockIdx.x] = scale;
+        } else {
+            scale = scale_io[0];
+        }
+        u32x2 *out = reinterpret_cast<u32x2 *>(norm_out) + row_base;
+        for (int c = tid; c < chunks_per_row; c += blockDim.x) {
+            const u32x4 v = normed(c);
+            float q[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                q[2 * j] = clamp_sym(P::lo(v[j]) / scale, fp8_max);
+                q[2 * j + 1] = clamp_sym(P::hi(v[j]) / scale, fp8_max);
+            }
+            out[c] = u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+        }
+    }
+}
+
+int g_force_nchunk = 0;  // 0 = heuristic; set through gpuk_set_tuning for sweeps
+
+// Chunks per lane.  Few rows (decode): spread a row over as many lanes as possible to shorten the
+// dependent chain.  Many rows: 4 chunks per lane keeps 8 independent 16-byte loads in flight per lane
+// with 256-lane workgroups at hidden 8192.
+int pick_nchunk(int64_t tokens, int chunks_per_row) {
+    auto fits = [&](int n) { return (int64_t)n * kMaxThreads >= chunks_per_row; };
+    if (g_force_nchunk) {
+        int n = g_force_nchunk;
+        while (n < 8 && !fits(n)) n *= 2;
+        return fits(n) ? n : 0;
+    }
+    int n = 1;
+    if (tokens > 256) {
+        if (chunks_per_row >= 1024) n = 4;
+        else if (chunks_per_row >= 256) n = 2;
+    } else if (tokens > 32) {
+        if (chunks_per_row >= 512) n = 2;
+    }
+    while (n < 8 && !fits(n)) n *= 2;
+    return fits(n) ? n : 0;
+}
+
+template <typename T, int QUANT>
+int launch(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
+           float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream) {
+    const int chunks = (int)(hidden / 8);
+    const int nchunk = pick_nchunk(tokens, chunks);
+    const dim3 grid((unsigned)tokens);
+    auto xs = static_cast<const u32x4 *>(x);
+    auto rs = static_cast<const u32x4 *>(residual_in);
+    auto gs = static_cast<const u32x4 *>(gamma);
+    auto ro = static_cast<u32x4 *>(residual_out);
+    const float hf = (float)hidden;
+    if (nchunk == 0) {
+        add_rmsnorm_quant_long_rows<T, QUANT><<<grid, kMaxThreads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale, chunks, hf, eps, fp8_max);
+        return hip_status(hipGetLastError());
+    }
+    const int threads = round_up((chunks + nchunk - 1) / nchunk, 64);
+#define GPUK_LAUNCH_NQ(N)                                                                                      \
+    case N:                                                                                                    \
+        add_rmsnorm_quant_rows<T, N, QUANT><<<grid, threads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale,     \
+                                                                          chunks, hf, eps, fp8_max);           \
+        break;
+    switch (nchunk) {
+        GPUK_LAUNCH_NQ(1)
+        GPUK_LAUNCH_NQ(2)
+        GPUK_LAUNCH_NQ(4)
+        GPUK_LAUNCH_NQ(8)
+        default: return GPUK_ERR_INTERNAL;
+    }
+#undef GPUK_LAUNCH_NQ
+    return hip_status(hipGetLastError());
+}
+
+template <typename T>
+int launch_quant(int quant_mode, const void *x, const void *residual_in, const void *gamma, void *residual_out,
+                 void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max,
+                 hipStream_t stream) {
+    switch (quant_mode) {
+        case GPUK_QUANT_NONE:
+            return launch<T, GPUK_QUANT_NONE>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+        case GPUK_QUANT_FP8_DYNAMIC:
+            return launch<T, GPUK_QUANT_FP8_DYNAMIC>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+        case GPUK_QUANT_FP8_STATIC:
+            return launch<T, GPUK_QUANT_FP8_STATIC>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+        default:
+            return GPUK_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace
+
+void set_norm_quant_nchunk(int n) { g_force_nchunk = n; }
+
+}  // namespace gpuk
+
+extern "C" int gpuk_add_rmsnorm_quant(const void *x, const void *residual_in, const void *gamma, void *residual_out,
+                                      void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps,
+                                      int dtype, int quant_mode, float fp8_max, void *stream) {
+    using namespace gpuk;
+    if (tokens < 0 || hidden <= 0) return GPUK_ERR_INVALID_ARG;
+    if (hidden % 8 != 0) return GPUK_ERR_UNSUPPORTED;           // rows are moved in 16-byte chunks
+    if (tokens > 0x7fffffffLL || hidden / 8 > 0x7fffffffLL) return GPUK_ERR_UNSUPPORTED;
+    if (!(fp8_max > 0.f) && quant_mode != GPUK_QUANT_NONE) return GPUK_ERR_INVALID_ARG;
+    if (quant_mode == GPUK_QUANT_FP8_E4M3FNUZ) return GPUK_ERR_UNSUPPORTED;  // gfx950 encodes OCP e4m3fn only
+    if (tokens == 0) return GPUK_OK;
+    if (!x || !residual_in || !gamma || !residual_out || !norm_out) return GPUK_ERR_INVALID_ARG;
+    if (quant_mode != GPUK_QUANT_NONE && !scale) return GPUK_ERR_INVALID_ARG;
+    if (!aligned16(x) || !aligned16(residual_in) || !aligned16(gamma) || !aligned16(residual_out)) return GPUK_ERR_MISALIGNED;
+    if (!(quant_mode == GPUK_QUANT_NONE ? aligned16(norm_out) : aligned8(norm_out))) return GPUK_ERR_MISALIGNED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case GPUK_DTYPE_BF16:
+            return launch_quant<BF16>(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
+        case GPUK_DTYPE_FP16:
+            return launch_quant<FP16>(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
+        default:
+            return GPUK_ERR_UNSUPPORTED;
+    }
+}

@@ -1,0 +1,34 @@
+// Entry points of the C ABI that launch nothing: status names, version, tuning knobs.
+#include <string.h>
+
+#include "../../../include/gpuk_amd.h"
+#include "host_utils.h"
+
+extern "C" const char *gpuk_status_string(int status) {
+    switch (status) {
+        case GPUK_OK: return "ok";
+        case GPUK_ERR_INVALID_ARG: return "invalid argument";
+        case GPUK_ERR_UNSUPPORTED: return "unsupported shape, dtype or mode";
+        case GPUK_ERR_MISALIGNED: return "pointer not aligned for vector access";
+        case GPUK_ERR_LAUNCH: return "kernel launch failed";
+        case GPUK_ERR_INTERNAL: return "internal error";
+        default: return "unknown status";
+    }
+}
+
+extern "C" int gpuk_abi_version(void) { return GPUK_AMD_ABI_VERSION; }
+
+extern "C" int gpuk_set_tuning(const char *key, int value) {
+    if (!key) return GPUK_ERR_INVALID_ARG;
+    if (strcmp(key, "norm_quant_nchunk") == 0) {
+        if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8) return GPUK_ERR_INVALID_ARG;
+        gpuk::set_norm_quant_nchunk(value);
+        return GPUK_OK;
+    }
+    if (strcmp(key, "rope_block_threads") == 0) {
+        if (value != 0 && value != 64 && value != 128 && value != 256 && value != 512) return GPUK_ERR_INVALID_ARG;
+        gpuk::set_rope_tuning(0, value);
+        return GPUK_OK;
+    }
+    return GPUK_ERR_INVALID_ARG;
+}

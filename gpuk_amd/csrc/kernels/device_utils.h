@@ -1,0 +1,129 @@
+// Device-side building blocks shared by the gfx950 kernels: 16-bit float pack/unpack on the
+// hardware converters, wave64 DPP reductions, and the OCP e4m3fn packed converter.
+//
+// Replaces the reference's src/common/kernel_utils.h (vec_t, 32-wide shuffle reductions,
+// block_reduce with WARP_SIZE hard-coded to 32: kernel_utils.h:29-53) and src/common/float8.h
+// (software fp32->fp8 encoder: float8.h:17-150) with wave64 / hardware equivalents.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gpuk {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+struct BF16 {};  // tag types: the 16-bit storage format of activations
+struct FP16 {};
+
+// Two 16-bit floats packed in one dword <-> two fp32 values.  Packing rounds to nearest even
+// (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32).
+template <typename T> struct Pack16;
+
+template <> struct Pack16<BF16> {
+    static __device__ __forceinline__ float lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        f32x2 v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+    }
+};
+
+template <> struct Pack16<FP16> {
+    static __device__ __forceinline__ float lo(uint32_t w) {
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+    }
+    static __device__ __forceinline__ float hi(uint32_t w) {
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+    }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        const uint32_t l = __builtin_bit_cast(uint16_t, (_Float16)a);
+        const uint32_t h = __builtin_bit_cast(uint16_t, (_Float16)b);
+        return l | (h << 16);
+    }
+};
+
+// ---- DPP lane exchange.  CTRL encodings: quad_perm[a,b,c,d] = a|b<<2|c<<4|d<<6,
+// row_half_mirror = 0x141, row_mirror = 0x140 (both reverse within 8 / 16 lanes).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __builtin_bit_cast(float,
+                              __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+constexpr int DPP_QUAD_XOR1 = 0xB1;       // quad_perm [1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;       // quad_perm [2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+constexpr int DPP_ROW_MIRROR = 0x140;
+
+struct SumOp {
+    static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
+};
+struct MaxOp {
+    static __device__ __forceinline__ float apply(float a, float b) { return __builtin_fmaxf(a, b); }
+};
+
+// All-reduce over aligned groups of LANES consecutive lanes (LANES in {4, 8, 16}): every lane
+// ends with its group's result.  One DPP row is 16 lanes, so these never leave the row.
+template <typename Op, int LANES>
+__device__ __forceinline__ float group_allreduce(float v) {
+    static_assert(LANES == 4 || LANES == 8 || LANES == 16, "group must fit in one DPP row");
+    v = Op::apply(v, dpp_f32<DPP_QUAD_XOR1>(v));
+    v = Op::apply(v, dpp_f32<DPP_QUAD_XOR2>(v));
+    if constexpr (LANES >= 8) v = Op::apply(v, dpp_f32<DPP_ROW_HALF_MIRROR>(v));
+    if constexpr (LANES >= 16) v = Op::apply(v, dpp_f32<DPP_ROW_MIRROR>(v));
+    return v;
+}
+
+// All-reduce over the 64 lanes of a wave; the result is wave-uniform.  Four row results are
+// combined in a fixed order (rows 0,1,2,3), so the value does not depend on lane.
+template <typename Op>
+__device__ __forceinline__ float wave_allreduce(float v) {
+    v = group_allreduce<Op, 16>(v);
+    int b = __builtin_bit_cast(int, v);
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return Op::apply(Op::apply(r0, r1), Op::apply(r2, r3));
+}
+
+// Workgroup all-reduce: wave results meet in LDS (one float per wave, at most 16 waves) and
+// every thread folds them in wave order.  `slots` must be private to this call site so that two
+// consecutive reductions need only one barrier each.
+template <typename Op>
+__device__ __forceinline__ float block_allreduce(float v, float *slots, int num_waves) {
+    v = wave_allreduce<Op>(v);
+    if (num_waves == 1) return v;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) slots[wave] = v;
+    __syncthreads();
+    float acc = slots[0];
+    for (int w = 1; w < num_waves; ++w) acc = Op::apply(acc, slots[w]);
+    return acc;
+}
+
+// Four fp32 -> four OCP e4m3fn codes in one dword (two v_cvt_pk_fp8_f32).  Inputs must already be
+// clamped to the finite range; rounding is to nearest even.
+__device__ __forceinline__ uint32_t cvt4_e4m3fn(float a, float b, float c, float d) {
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+    return (uint32_t)w;
+}
+
+__device__ __forceinline__ float clamp_sym(float v, float bound) {
+    return __builtin_amdgcn_fmed3f(v, -bound, bound);
+}
+
+// Correctly rounded fp32 quotient a/b given rcp = RN(1/b): one multiply and two fused
+// multiply-adds (Markstein's correction step).  Valid while a/b, the residual and rcp stay in the
+// normal range; callers guard the range of b once per row and fall back to `/` outside it.
+__device__ __forceinline__ float div_by_rcp(float a, float b, float rcp) {
+    float q = a * rcp;
+    float e = __builtin_fmaf(-q, b, a);
+    return __builtin_fmaf(e, rcp, q);
+}
+
+}  // namespace gpuk

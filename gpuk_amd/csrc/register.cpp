@@ -1,0 +1,47 @@
+// Operator registration of the `gpuk` torch library for the two fused paths.
+//
+// The four schema strings marked "reference" are the reference's own (src/register.cpp:37-39, :42-44,
+// :47-49, :52-55), so `torch.ops.gpuk.<name>(...)` call sites keep working unchanged.  Compute ops are
+// registered for the CUDA dispatch key, which is the key HIP tensors carry on PyTorch-ROCm.
+#include "ops/ops.h"
+
+TORCH_LIBRARY(gpuk, m) {
+    using namespace gpuk_ops;
+
+    // reference: src/register.cpp:37-40
+    m.def("allreduce_rms(SymInt fptr, Tensor allreduce_in, Tensor residual_in, Tensor rms_gamma, Tensor residual_out, "
+          "Tensor norm_out, Tensor scale_out, float eps, SymInt quant_type) -> ()");
+    m.impl("allreduce_rms", c10::DispatchKey::CUDA, &allreduce_rms);
+
+    // reference: src/register.cpp:42-45
+    m.def("fused_rope_rms(Tensor qkv, Tensor qw, Tensor kw, Tensor cos_sin, Tensor positions, SymInt num_tokens, "
+          "SymInt num_heads_q, SymInt num_heads_k, SymInt num_heads_v, SymInt head_size, bool is_neox_style, "
+          "float eps) -> ()");
+    m.impl("fused_rope_rms", c10::DispatchKey::CUDA, &fused_rope_rms);
+
+    // reference: src/register.cpp:47-50
+    m.def("fused_mrope_3d_rms(Tensor qkv, Tensor qw, Tensor kw, Tensor cos_sin, Tensor positions, SymInt num_tokens, "
+          "SymInt num_heads_q, SymInt num_heads_k, SymInt num_heads_v, SymInt head_size, bool is_neox_style, "
+          "int[] mrope_section_, bool is_interleaved, float eps) -> ()");
+    m.impl("fused_mrope_3d_rms", c10::DispatchKey::CUDA, &fused_mrope_3d_rms);
+
+    // reference: src/register.cpp:52-56
+    m.def("fused_mrope_3d_rms_set_kv(Tensor qkv, Tensor qw, Tensor kw, Tensor cos_sin, Tensor positions, "
+          "SymInt num_tokens, SymInt num_heads_q, SymInt num_heads_k, SymInt num_heads_v, SymInt head_size, "
+          "bool is_neox_style, int[] mrope_section_, bool is_interleaved, float eps, Tensor q, Tensor k_cache, "
+          "Tensor v_cache, Tensor kv_loc, float k_scale, float v_scale) -> ()");
+    m.impl("fused_mrope_3d_rms_set_kv", c10::DispatchKey::CUDA, &fused_mrope_3d_rms_set_kv);
+
+    // additive: plain-RoPE form of the KV-writing op (1-D positions)
+    m.def("fused_rope_rms_set_kv(Tensor qkv, Tensor qw, Tensor kw, Tensor cos_sin, Tensor positions, "
+          "SymInt num_tokens, SymInt num_heads_q, SymInt num_heads_k, SymInt num_heads_v, SymInt head_size, "
+          "bool is_neox_style, float eps, Tensor q, Tensor k_cache, Tensor v_cache, Tensor kv_loc, float k_scale, "
+          "float v_scale) -> ()");
+    m.impl("fused_rope_rms_set_kv", c10::DispatchKey::CUDA, &fused_rope_rms_set_kv);
+
+    // additive: amax divisor / clamp bound of the fp8 modes of allreduce_rms (448 OCP default, 240 reference)
+    m.def("set_fp8_max(float value) -> ()");
+    m.impl("set_fp8_max", &set_fp8_max);
+    m.def("get_fp8_max() -> float");
+    m.impl("get_fp8_max", &get_fp8_max);
+}

@@ -1,0 +1,133 @@
+/*
+ * gpuk_amd.h -- C ABI of libgpuk_amd.so: gfx950 (MI355X) kernels for gpuk's memory-bound fused
+ * inference ops.  Plain pointers and sizes, no torch types, no exceptions, no ownership transfer:
+ * every buffer is borrowed for the duration of the enqueued kernel.  All entry points are
+ * asynchronous on `stream` (a hipStream_t passed as void*; NULL = the default stream), allocate
+ * nothing and never synchronise, so they can be recorded into a HIP graph.
+ *
+ * Each function returns GPUK_OK (0) or a gpuk_status; gpuk_status_string() names it.
+ * Device pointers must be 16-byte aligned (8-byte for fp8 code buffers) as noted per argument.
+ *
+ * The reference interface each entry point stands behind is cited as <file>:<lines> in the
+ * reference repository (xytpai/gpuk).
+ */
+#ifndef GPUK_AMD_H_
+#define GPUK_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GPUK_AMD_ABI_VERSION 1
+
+typedef enum gpuk_status {
+    GPUK_OK = 0,
+    GPUK_ERR_INVALID_ARG = 1,  /* null pointer, negative size, inconsistent sections ...        */
+    GPUK_ERR_UNSUPPORTED = 2,  /* a shape / dtype / mode this build has no kernel for            */
+    GPUK_ERR_MISALIGNED = 3,   /* a pointer misses the alignment the vector accesses need         */
+    GPUK_ERR_LAUNCH = 4,       /* hipGetLastError() reported a launch failure                     */
+    GPUK_ERR_INTERNAL = 5
+} gpuk_status;
+
+/* 16-bit activation formats (the reference dispatches on at::ScalarType:
+ * src/ops/all_reduce_fusion.cpp:375, src/ops/fused_rope.cpp:27-31). */
+typedef enum gpuk_dtype {
+    GPUK_DTYPE_BF16 = 0,
+    GPUK_DTYPE_FP16 = 1
+} gpuk_dtype;
+
+/* quant_type of the allreduce_rms op.  0/1/2 are the reference's QuantType
+ * (src/impl/all_reduce_fusion_impl.h:13-17); 3 is additive. */
+typedef enum gpuk_quant {
+    GPUK_QUANT_NONE = 0,         /* norm_out holds the activation dtype                                   */
+    GPUK_QUANT_FP8_DYNAMIC = 1,  /* e4m3fn codes, per-token scale written to scale[tokens]                */
+    GPUK_QUANT_FP8_E4M3FNUZ = 2, /* MI300 fnuz encoding: rejected with GPUK_ERR_UNSUPPORTED on gfx950     */
+    GPUK_QUANT_FP8_STATIC = 3    /* e4m3fn codes, one per-tensor scale read from scale[0]                 */
+} gpuk_quant;
+
+/* Storage format of the paged KV cache. */
+typedef enum gpuk_kv_dtype {
+    GPUK_KV_SAME = 0,   /* cache holds the activation dtype; K/V are stored unscaled
+                           (src/impl/rope_rms_impl.h:213-214,225-226)                                    */
+    GPUK_KV_E4M3FN = 1  /* cache holds e4m3fn codes of x / scale (src/impl/rope_rms_impl.h:109-118,215-217) */
+} gpuk_kv_dtype;
+
+const char *gpuk_status_string(int status);
+int gpuk_abi_version(void);
+
+/*
+ * residual_out = x + residual_in ; norm_out = quant(RMSNorm(residual_out) * gamma).
+ *
+ * Stands behind the allreduce_rms op for the one-GPU case (no all-reduce):
+ * host op src/ops/all_reduce_fusion.cpp:363-396, launcher src/impl/all_reduce_fusion_impl.h:424-469,
+ * device code :256-265 (residual add) + :202-228 (epilogue).  Rounding follows the reference's torch
+ * oracle gpuk/__init__.py:147-164.
+ *
+ *   x, residual_in, residual_out : [tokens, hidden] contiguous, `dtype`, 16-byte aligned
+ *   gamma                        : [hidden] `dtype`, 16-byte aligned
+ *   norm_out                     : [tokens, hidden]; `dtype` (16-byte aligned) for GPUK_QUANT_NONE,
+ *                                  else one byte per element (8-byte aligned)
+ *   scale                        : fp32; written [tokens] for FP8_DYNAMIC, read [1] for FP8_STATIC,
+ *                                  ignored (may be NULL) for NONE
+ *   hidden                       : multiple of 8 (the reference supports 1024/2048/4096 only:
+ *                                  all_reduce_fusion_impl.h:389-401)
+ *   fp8_max                      : clamp bound and amax divisor; 448 (OCP e4m3fn) or 240 (the
+ *                                  reference's fp8e4m3fn::max_value, src/common/float8.h:216-218)
+ */
+int gpuk_add_rmsnorm_quant(const void *x, const void *residual_in, const void *gamma, void *residual_out,
+                           void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps, int dtype,
+                           int quant_mode, float fp8_max, void *stream);
+
+/*
+ * Per-head RMSNorm of Q and K, then rotary embedding, written back in place; V is not touched.
+ *
+ * Stands behind fused_rope_rms (src/ops/fused_rope.cpp:19-49 -> src/impl/rope_rms_impl.h:468-503)
+ * with n_axes == 1 and behind fused_mrope_3d_rms (fused_rope.cpp:51-89 -> rope_rms_impl.h:505-555)
+ * with n_axes == 3.  Rounding follows test/test_fused_rope_rms.py:8-34.
+ *
+ *   qkv        : [num_tokens, hq+hk+hv, head_size] contiguous `dtype`, 16-byte aligned, in/out
+ *   qw, kw     : [head_size] `dtype`
+ *   cos_sin    : [max_positions, head_size] `dtype`; row p = cos(p*f_0..f_{D/2-1}) | sin(...)
+ *   positions  : int64; element (axis a, token t) at positions[a*pos_stride_axis + t*pos_stride_token]
+ *   n_axes     : 1 (RoPE) or 3 (mRoPE; mrope_section[3] sums to head_size/2)
+ *   interleaved: mRoPE frequency->axis map; 0 chunked, 1 interleaved (rope_rms_impl.h:120-153)
+ *   head_size  : 64, 128 or 256 (rope_rms_impl.h:473)
+ */
+int gpuk_rope_rms(void *qkv, const void *qw, const void *kw, const void *cos_sin, const int64_t *positions,
+                  int64_t pos_stride_axis, int64_t pos_stride_token, int n_axes, int64_t num_tokens,
+                  int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v, int64_t head_size,
+                  int is_neox_style, const int64_t *mrope_section, int is_interleaved, float eps, int dtype,
+                  void *stream);
+
+/*
+ * Same arithmetic, results scattered: q -> q_out[t,h,:], k -> k_cache[kv_loc[t],h,:],
+ * v -> v_cache[kv_loc[t],h,:]; qkv is read only.
+ *
+ * Stands behind fused_mrope_3d_rms_set_kv (src/ops/fused_rope.cpp:91-166 ->
+ * src/impl/rope_rms_impl.h:557-610, kernels :157-301) with n_axes == 3; n_axes == 1 is the additive
+ * fused_rope_rms_set_kv.  Rounding follows test/test_fused_mrope_rms_set_kv.py:62-130.
+ *
+ *   q_out            : [num_tokens, hq, head_size] `dtype`, 16-byte aligned
+ *   k_cache, v_cache : [slots, hk|hv, head_size]; `dtype` or e4m3fn bytes per kv_dtype; slots not named
+ *                      by kv_loc are left bit-identical
+ *   kv_loc           : [num_tokens] int64 slot per token (duplicates race; last writer wins)
+ *   k_scale, v_scale : used only with GPUK_KV_E4M3FN: code = e4m3fn(rT(x / scale)), saturating at +-448
+ */
+int gpuk_rope_rms_set_kv(const void *qkv, const void *qw, const void *kw, const void *cos_sin,
+                         const int64_t *positions, int64_t pos_stride_axis, int64_t pos_stride_token, int n_axes,
+                         int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                         int64_t head_size, int is_neox_style, const int64_t *mrope_section, int is_interleaved,
+                         float eps, int dtype, void *q_out, void *k_cache, void *v_cache, const int64_t *kv_loc,
+                         float k_scale, float v_scale, int kv_dtype, void *stream);
+
+/* Development knob for sweeps: key "norm_quant_nchunk" (0 = heuristic, else 1/2/4/8 chunks per lane),
+ * "rope_heads_per_wave" ... Unknown keys return GPUK_ERR_INVALID_ARG.  Not part of the reference. */
+int gpuk_set_tuning(const char *key, int value);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* GPUK_AMD_H_ */

@@ -1,0 +1,251 @@
+"""GPU parity: fused QK-RMSNorm + RoPE / mRoPE (+ paged KV-cache write) against the CPU restatement of
+the reference's torch oracle on the same seeded inputs, through the C ABI and through the torch ops.
+
+The shape sweep follows the reference's own test scripts (test/test_fused_rope_rms.py:196-217,
+test/test_fused_mrope_rms_set_kv.py:274-307): NeoX and GPT-J style, odd token counts, head sizes
+64/128/256 with mRoPE sections [12,10,10] / [24,20,20] / [48,40,40], chunked and interleaved, a random
+cos/sin table, fp8 cache with k_scale 1.5 and v_scale 2.0 -- but with distinct cache slots, so the result
+is deterministic.
+"""
+import pytest
+import torch
+
+from gpuk_amd import workloads
+from oracle import c_oracle, torch_oracle as O
+from tests.util import assert_bits_equal, assert_codes_close, assert_rotated_close
+
+pytestmark = pytest.mark.gpu
+
+SECTIONS = {64: [12, 10, 10], 128: [24, 20, 20], 256: [48, 40, 40]}
+
+
+def to_dev(inp, device):
+    return [t.to(device) for t in (inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, inp.kv_loc)]
+
+
+def oracle_inplace(inp):
+    q, k, v = O.rope_rms_ref(inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, inp.num_tokens, inp.num_heads_q,
+                             inp.num_heads_k, inp.num_heads_v, inp.head_size, inp.is_neox, inp.eps,
+                             inp.mrope_section, inp.is_interleaved)
+    return torch.cat([q, k, v], dim=1)
+
+
+def run_inplace(inp, device):
+    from gpuk_amd import capi
+
+    qkv, qw, kw, cs, pos, _ = to_dev(inp, device)
+    capi.rope_rms(qkv, qw, kw, cs, pos, inp.num_tokens, inp.num_heads_q, inp.num_heads_k, inp.num_heads_v,
+                  inp.head_size, inp.is_neox, inp.eps, inp.mrope_section, inp.is_interleaved)
+    torch.cuda.synchronize()
+    return qkv
+
+
+def run_set_kv(inp, device, via_op=False):
+    qkv, qw, kw, cs, pos, loc = to_dev(inp, device)
+    k0, v0 = inp.new_cache()
+    kc, vc = k0.to(device), v0.to(device)
+    q_out = torch.empty((inp.num_tokens, inp.num_heads_q, inp.head_size), dtype=qkv.dtype, device=device)
+    args = (qkv, qw, kw, cs, pos, inp.num_tokens, inp.num_heads_q, inp.num_heads_k, inp.num_heads_v, inp.head_size,
+            inp.is_neox)
+    if via_op:
+        import gpuk_amd as gpuk
+
+        if inp.mrope_section is not None:
+            gpuk.fused_mrope_3d_rms_set_kv(*args, inp.mrope_section, inp.is_interleaved, inp.eps, q_out, kc, vc, loc,
+                                           inp.k_scale, inp.v_scale)
+        else:
+            gpuk.fused_rope_rms_set_kv(*args, inp.eps, q_out, kc, vc, loc, inp.k_scale, inp.v_scale)
+    else:
+        from gpuk_amd import capi
+
+        capi.rope_rms_set_kv(*args, inp.eps, q_out, kc, vc, loc, inp.k_scale, inp.v_scale, inp.mrope_section,
+                             inp.is_interleaved)
+    torch.cuda.synchronize()
+    assert torch.equal(qkv.cpu(), inp.qkv), "set_kv must not modify qkv"
+    return q_out, kc, vc, (k0, v0)
+
+
+def check_set_kv(inp, got, tag):
+    q_out, kc, vc, (k0, v0) = got
+    q_ref = torch.empty_like(q_out, device="cpu")
+    k_ref, v_ref = k0.clone(), v0.clone()
+    O.rope_rms_set_kv_ref(inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, inp.num_tokens, inp.num_heads_q,
+                          inp.num_heads_k, inp.num_heads_v, inp.head_size, inp.is_neox, inp.eps, q_ref, k_ref, v_ref,
+                          inp.kv_loc, inp.k_scale, inp.v_scale, inp.mrope_section, inp.is_interleaved)
+    assert_rotated_close(q_out, q_ref, f"{tag} q_out")
+    kc, vc = kc.cpu(), vc.cpu()
+    loc = inp.kv_loc
+    if inp.kv_dtype == torch.float8_e4m3fn:
+        assert_codes_close(kc[loc], k_ref[loc], f"{tag} k_cache codes")
+        assert_bits_equal(vc[loc].view(torch.uint8), v_ref[loc].view(torch.uint8), f"{tag} v_cache codes")
+    else:
+        assert_rotated_close(kc[loc], k_ref[loc], f"{tag} k_cache")
+        assert_bits_equal(vc[loc], v_ref[loc], f"{tag} v_cache")
+    untouched = torch.ones(inp.num_slots, dtype=torch.bool)
+    untouched[loc] = False
+    assert_bits_equal(kc[untouched].view(torch.uint8), k0[untouched].view(torch.uint8), f"{tag} untouched k slots")
+    assert_bits_equal(vc[untouched].view(torch.uint8), v0[untouched].view(torch.uint8), f"{tag} untouched v slots")
+
+
+def make(tokens, heads, head_size, neox, seed, mrope=False, interleaved=False, fp8=False, hk=None, hv=None):
+    inp = workloads.rope_inputs(tokens, heads, heads if hk is None else hk, heads if hv is None else hv, head_size,
+                                seed=seed, max_pos=10000, num_slots=max(2 * tokens, 64), is_neox=neox,
+                                random_table=True,
+                                kv_dtype=torch.float8_e4m3fn if fp8 else torch.bfloat16,
+                                k_scale=1.5 if fp8 else 1.0, v_scale=2.0 if fp8 else 1.0)
+    if mrope:
+        g = torch.Generator().manual_seed(seed + 1)
+        inp.positions = torch.randint(0, 10000, (3, tokens), generator=g, dtype=torch.int64)
+        inp.mrope_section = SECTIONS[head_size]
+        inp.is_interleaved = interleaved
+    return inp
+
+
+@pytest.mark.parametrize("neox", [True, False])
+@pytest.mark.parametrize("tokens", [513, 127, 3])
+@pytest.mark.parametrize("head_size", [64, 128, 256])
+def test_rope_inplace_sweep(device, neox, tokens, head_size):
+    print(f"case inplace neox={neox} T={tokens} D={head_size}", flush=True)
+    inp = make(tokens, 32, head_size, neox, seed=tokens + head_size)
+    got = run_inplace(inp, device)
+    want = oracle_inplace(inp)
+    nqk = inp.num_heads_q + inp.num_heads_k
+    assert_rotated_close(got[:, :nqk], want[:, :nqk], "q,k")
+    assert_bits_equal(got[:, nqk:], want[:, nqk:], "v untouched")
+
+
+@pytest.mark.parametrize("neox", [True, False])
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("head_size", [64, 128, 256])
+def test_mrope_inplace_sweep(device, neox, interleaved, head_size):
+    print(f"case mrope inplace neox={neox} il={interleaved} D={head_size}", flush=True)
+    inp = make(257, 32, head_size, neox, seed=7 + head_size, mrope=True, interleaved=interleaved)
+    got = run_inplace(inp, device)
+    want = oracle_inplace(inp)
+    nqk = inp.num_heads_q + inp.num_heads_k
+    assert_rotated_close(got[:, :nqk], want[:, :nqk], "q,k")
+    assert_bits_equal(got[:, nqk:], want[:, nqk:], "v untouched")
+
+
+@pytest.mark.parametrize("neox", [True, False])
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("head_size", [64, 128, 256])
+@pytest.mark.parametrize("fp8", [True, False])
+def test_mrope_set_kv_sweep(device, neox, interleaved, head_size, fp8):
+    print(f"case mrope set_kv neox={neox} il={interleaved} D={head_size} fp8={fp8}", flush=True)
+    inp = make(131, 32, head_size, neox, seed=17 + head_size, mrope=True, interleaved=interleaved, fp8=fp8)
+    check_set_kv(inp, run_set_kv(inp, device), "[mrope set_kv]")
+
+
+@pytest.mark.parametrize("hq,hk,hv", [(32, 8, 8), (28, 4, 4), (64, 8, 8), (5, 3, 2), (1, 1, 1), (40, 40, 40)])
+@pytest.mark.parametrize("fp8", [True, False])
+def test_rope_set_kv_head_mixes(device, hq, hk, hv, fp8):
+    """GQA head mixes, including counts that do not fill a wave's group of heads."""
+    print(f"case set_kv heads={hq},{hk},{hv} fp8={fp8}", flush=True)
+    inp = make(67, hq, 128, True, seed=hq * 100 + hk, fp8=fp8, hk=hk, hv=hv)
+    check_set_kv(inp, run_set_kv(inp, device), f"[set_kv {hq},{hk},{hv}]")
+
+
+def test_config3_qwen3_like(device):
+    inp = workloads.config3()
+    check_set_kv(inp, run_set_kv(inp, device), "[C3]")
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_config4_qwen2vl_like(device, interleaved):
+    inp = workloads.config4(is_interleaved=interleaved)
+    check_set_kv(inp, run_set_kv(inp, device), f"[C4 il={interleaved}]")
+
+
+@pytest.mark.parametrize("tokens", workloads.DECODE_TOKENS)
+def test_config5_decode_fp8_cache(device, tokens):
+    inp = workloads.config5_rope(tokens)
+    check_set_kv(inp, run_set_kv(inp, device), f"[C5 T={tokens}]")
+
+
+def test_torch_ops(device):
+    """The drop-in path: torch.ops.gpuk.* with the reference's argument order."""
+    import gpuk_amd as gpuk
+
+    inp = make(97, 16, 128, True, seed=5)
+    qkv, qw, kw, cs, pos, _ = to_dev(inp, device)
+    gpuk.fused_rope_rms(qkv, qw, kw, cs, pos, inp.num_tokens, 16, 16, 16, 128, True, inp.eps)
+    torch.cuda.synchronize()
+    want = oracle_inplace(inp)
+    assert_rotated_close(qkv[:, :32], want[:, :32], "op fused_rope_rms q,k")
+    assert_bits_equal(qkv[:, 32:], want[:, 32:], "op fused_rope_rms v")
+
+    inp = make(97, 16, 128, False, seed=6, mrope=True, interleaved=True)
+    qkv, qw, kw, cs, pos, _ = to_dev(inp, device)
+    gpuk.fused_mrope_3d_rms(qkv, qw, kw, cs, pos, inp.num_tokens, 16, 16, 16, 128, False, inp.mrope_section, True,
+                            inp.eps)
+    torch.cuda.synchronize()
+    want = oracle_inplace(inp)
+    assert_rotated_close(qkv[:, :32], want[:, :32], "op fused_mrope_3d_rms q,k")
+
+    inp = make(97, 16, 128, True, seed=8, mrope=True, fp8=True)
+    check_set_kv(inp, run_set_kv(inp, device, via_op=True), "[op mrope set_kv fp8]")
+    inp = make(97, 16, 128, True, seed=9)
+    check_set_kv(inp, run_set_kv(inp, device, via_op=True), "[op rope set_kv bf16]")
+
+
+def test_strided_positions(device):
+    """positions is passed by stride (src/ops/fused_rope.cpp:104,121-122): a [T,3] buffer viewed as [3,T]."""
+    import gpuk_amd as gpuk
+
+    inp = make(65, 8, 128, True, seed=12, mrope=True)
+    pos_t = inp.positions.t().contiguous()          # [T,3] storage
+    inp.positions = pos_t.t()                        # [3,T] view with strides (1,3)
+    assert not inp.positions.is_contiguous()
+    qkv, qw, kw, cs, _, _ = to_dev(inp, device)
+    pos = pos_t.to(device).t()
+    gpuk.fused_mrope_3d_rms(qkv, qw, kw, cs, pos, 65, 8, 8, 8, 128, True, inp.mrope_section, False, inp.eps)
+    torch.cuda.synchronize()
+    want = oracle_inplace(inp)
+    assert_rotated_close(qkv[:, :16], want[:, :16], "strided positions q,k")
+
+
+def test_equal_axes_equal_plain_rope(device):
+    """mRoPE with three identical position rows selects the same table row everywhere: plain RoPE."""
+    inp = make(50, 8, 128, True, seed=13)
+    plain = run_inplace(inp, device)
+    inp.positions = inp.positions.unsqueeze(0).expand(3, -1).contiguous()
+    inp.mrope_section = [24, 20, 20]
+    for il in (False, True):
+        inp.is_interleaved = il
+        assert_bits_equal(run_inplace(inp, device), plain, f"mrope(equal axes, il={il}) vs rope")
+
+
+def test_fp16_activations(device):
+    inp = workloads.rope_inputs(33, 8, 4, 4, 128, seed=14, max_pos=4096, num_slots=128, dtype=torch.float16,
+                                random_table=True)
+    got = run_inplace(inp, device)
+    want = oracle_inplace(inp)
+    assert_rotated_close(got[:, :12], want[:, :12], "fp16 q,k")
+
+
+def test_matches_c_checker(device):
+    inp = make(40, 8, 128, False, seed=15, mrope=True, interleaved=True, fp8=True)
+    q_out, kc, vc, (k0, v0) = run_set_kv(inp, device)
+    q_ref = torch.empty_like(q_out, device="cpu")
+    k_ref, v_ref = k0.clone(), v0.clone()
+    c_oracle.rope_rms(inp.qkv.clone(), inp.qw, inp.kw, inp.cos_sin, inp.positions, 40, 8, 8, 8, 128, False, inp.eps,
+                      inp.mrope_section, True, q_ref, k_ref.view(torch.uint8), v_ref.view(torch.uint8), inp.kv_loc,
+                      inp.k_scale, inp.v_scale)
+    assert_rotated_close(q_out, q_ref, "q vs C")
+    assert_codes_close(kc.cpu(), k_ref, "k codes vs C")
+    assert_bits_equal(vc.cpu().view(torch.uint8), v_ref.view(torch.uint8), "v codes vs C")
+
+
+def test_op_rejects_bad_arguments(device):
+    import gpuk_amd as gpuk
+
+    inp = make(8, 4, 128, True, seed=16)
+    qkv, qw, kw, cs, pos, _ = to_dev(inp, device)
+    with pytest.raises(RuntimeError):   # 2-D positions for the 1-axis op (reference: TORCH_CHECK fused_rope.cpp:26)
+        gpuk.fused_rope_rms(qkv, qw, kw, cs, pos.unsqueeze(0), 8, 4, 4, 4, 128, True, 1e-6)
+    with pytest.raises(RuntimeError):   # sections must sum to head_size/2 (reference: assert rope_rms_impl.h:513)
+        gpuk.fused_mrope_3d_rms(qkv, qw, kw, cs, pos.unsqueeze(0).expand(3, -1).contiguous(), 8, 4, 4, 4, 128, True,
+                                [16, 16, 16], False, 1e-6)
+    with pytest.raises(RuntimeError):   # unsupported head size (reference: assert rope_rms_impl.h:473)
+        gpuk.fused_rope_rms(qkv, qw, kw, cs, pos, 8, 4, 4, 4, 96, True, 1e-6)
