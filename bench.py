@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused residual-add + RMSNorm + per-token FP8 quant path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A step is one call of `torch.ops.gpuk.allreduce_rms` (quant_type 1, no all-reduce) over one 8192 x 8192
+bf16 batch with 1 % +-50 outliers, inputs resident in HBM.  Buffers rotate over three distinct sets so no
+cache can serve a repeat.  Prints ONE JSON line:
+
+  value      achieved HBM GB/s over the K timed steps = algorithmic bytes (7*T*H + 4*T + 2*H) / wall time
+  roofline   the same kernel timed per launch with HIP events on the launch stream, against 8 TB/s
+  cpu_baseline  the restated torch reference on the host's cores, on a bounded row sample of the same batch
+  extras     secondary figures: copy-kernel ceiling, the RoPE + KV-write kernel on its two configurations,
+             decode-shape latencies (us/call)
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import re
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--tokens", type=int, default=8192)
+    ap.add_argument("--hidden", type=int, default=8192)
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the batch the CPU baseline runs on")
+    return ap.parse_args()
+
+
+def event_time_ms(fn, iters, warmup=3):
+    """Average duration of fn() in ms from HIP events on the current stream (where fn launches)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(iters):
+        fn(i)
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def per_launch_ms(fn, iters):
+    """Per-launch durations: one event pair around every launch, averaged."""
+    import torch
+
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(evs):
+        a.record()
+        fn(i)
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
+
+
+def traffic_from_profile(name):
+    """HBM bytes per launch measured with rocprofv3 counters, if a summary for this workload is committed."""
+    path = os.path.join(ROOT, "profiles", name)
+    if not os.path.exists(path):
+        return None
+    m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), re.M)
+    return float(m.group(1)) if m else None
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this benchmark is a single-GPU kernel measurement; --gpus {args.gpus} is not supported "
+              "(rows shard trivially across GPUs, no collective is involved)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import gpuk_amd as gpuk
+    from gpuk_amd import capi, workloads
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    T, H = args.tokens, args.hidden
+
+    # ------------------------------------------------------------------ primary: add + RMSNorm + per-token fp8
+    inp = workloads.config2(T, H)
+    NSETS = 3
+    sets = []
+    for s in range(NSETS):
+        x = inp.x.to(dev) if s == 0 else torch.roll(sets[0][0], shifts=s, dims=0).contiguous()
+        r = inp.residual.to(dev) if s == 0 else torch.roll(sets[0][1], shifts=s, dims=0).contiguous()
+        sets.append((x, r, torch.empty_like(x), torch.empty((T, H), dtype=torch.float8_e4m3fn, device=dev),
+                     torch.empty((T, 1), dtype=torch.float32, device=dev)))
+    gamma = inp.gamma.to(dev)
+    eps = inp.eps
+    alg_bytes = workloads.norm_quant_bytes(T, H, quant=1)
+
+    def step(i=0):
+        x, r, ro, codes, sc = sets[i % NSETS]
+        gpuk.allreduce_rms(0, x, r, gamma, ro, codes, sc, eps, gpuk.QUANT_FP8_DYNAMIC)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = alg_bytes / (wall / args.steps) / 1e9
+
+    avg_ms, med_ms, min_ms = per_launch_ms(step, min(args.steps, 200))
+    achieved = alg_bytes / (avg_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": traffic_from_profile("add_rmsnorm_quant_8192x8192.md"),
+                "kernel": "add_rmsnorm_quant_rows<BF16,4,dynamic>", "avg_launch_us": round(avg_ms * 1e3, 2),
+                "median_launch_us": round(med_ms * 1e3, 2), "min_launch_us": round(min_ms * 1e3, 2),
+                "algorithmic_bytes": alg_bytes}
+
+    # ------------------------------------------------------------------ CPU baseline (bounded sample)
+    cpu_baseline = None
+    if not args.no_cpu:
+        from oracle import torch_oracle as O
+
+        rows = min(args.cpu_rows, T)
+        ncores = os.cpu_count() or 1
+        threads = int(os.environ.get("OMP_NUM_THREADS", ncores))
+        torch.set_num_threads(threads)
+        xs, rs = inp.x[:rows], inp.residual[:rows]
+        O.add_rmsnorm_quant_ref(xs, rs, inp.gamma, eps, O.QUANT_DYNAMIC)
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            O.add_rmsnorm_quant_ref(xs, rs, inp.gamma, eps, O.QUANT_DYNAMIC)
+            times.append(time.perf_counter() - t0)
+        t_med = sorted(times)[1]
+        cpu_baseline = {"value": round(workloads.norm_quant_bytes(rows, H, 1) / t_med / 1e9, 3), "unit": "GB/s",
+                        "cores": torch.get_num_threads(), "kind": "port",
+                        "sample": f"restated torch reference on CPU tensors, first {rows} of {T} rows x {H}, "
+                                  f"median of 3 calls ({t_med * 1e3:.0f} ms/call); host reports {ncores} cpus"}
+
+    # ------------------------------------------------------------------ secondary figures
+    extras = {}
+    if not args.no_extras:
+        # practical ceiling: plain copy, 512 MiB in + 512 MiB out
+        nb = 512 << 20
+        src = torch.empty(nb, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        cp_ms = event_time_ms(lambda i=0: capi.copy_bytes(dst, src, nb), 20)
+        extras["copy_kernel_GBps"] = round(2 * nb / (cp_ms * 1e-3) / 1e9, 1)
+        del src, dst
+
+        def rope_case(r, n_sets):
+            n_axes = 3 if r.mrope_section is not None else 1
+            kv_elem = 1 if r.kv_dtype == torch.float8_e4m3fn else 2
+            nbytes = workloads.rope_set_kv_bytes(r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v,
+                                                 r.head_size, n_axes, kv_elem)
+            k0, v0 = r.new_cache()
+            qw, kw, cs, pos, loc = (t.to(dev) for t in (r.qw, r.kw, r.cos_sin, r.positions, r.kv_loc))
+            bufs = []
+            for s in range(n_sets):
+                bufs.append((r.qkv.to(dev).clone(), torch.empty((r.num_tokens, r.num_heads_q, r.head_size),
+                                                                 dtype=torch.bfloat16, device=dev),
+                             k0.to(dev), v0.to(dev)))
+
+            def call(i=0):
+                qkv, q_out, kc, vc = bufs[i % n_sets]
+                capi.rope_rms_set_kv(qkv, qw, kw, cs, pos, r.num_tokens, r.num_heads_q, r.num_heads_k,
+                                     r.num_heads_v, r.head_size, r.is_neox, r.eps, q_out, kc, vc, loc, r.k_scale,
+                                     r.v_scale, r.mrope_section, r.is_interleaved)
+
+            avg, med, mn = per_launch_ms(call, 100)
+            burst = event_time_ms(call, 100)
+            return nbytes, avg, med, mn, burst
+
+        for name, r in (("rope_kv_qwen3_T4096", workloads.config3()), ("mrope_kv_qwen2vl_T8192", workloads.config4())):
+            nbytes, avg, med, mn, burst = rope_case(r, 4)
+            extras[name] = {"us_per_call": round(burst * 1e3, 2), "avg_launch_us": round(avg * 1e3, 2),
+                            "GBps": round(nbytes / (burst * 1e-3) / 1e9, 1),
+                            "frac_of_8TBps": round(nbytes / (burst * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                            "algorithmic_bytes": nbytes}
+
+        decode = {}
+        for t in workloads.DECODE_TOKENS:
+            d = workloads.config5_norm(t)
+            x, r_, g = d.x.to(dev), d.residual.to(dev), d.gamma.to(dev)
+            ro = torch.empty_like(x)
+            codes = torch.empty((t, 7168), dtype=torch.float8_e4m3fn, device=dev)
+            sc = torch.empty((t, 1), dtype=torch.float32, device=dev)
+            a_ms = event_time_ms(lambda i=0: capi.add_rmsnorm_quant(x, r_, g, ro, codes, sc, d.eps, 1), 300)
+            nbytes, avg, med, mn, burst = rope_case(workloads.config5_rope(t), 2)
+            decode[str(t)] = {"add_rmsnorm_quant_us": round(a_ms * 1e3, 2), "rope_kv_fp8_us": round(burst * 1e3, 2)}
+        extras["decode_us_per_call"] = decode
+
+    out = {
+        "metric": "HBM GB/s add+RMSNorm+FP8 per-token quant @8192x8192 bf16",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"residual-add + RMSNorm + dynamic per-token e4m3fn quant, tokens={T}, hidden={H}, "
+                               "bf16, x~N(0,1), residual~N(0,sigma=2), gamma~N(1,0.1), 1% of x = +-50, eps=1e-6",
+                   "entry": "torch.ops.gpuk.allreduce_rms(fptr=0, quant_type=1)", "buffer_sets": NSETS},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "extras": extras,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -28,7 +28,7 @@ ARCH = "gfx950"
 DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-ffp-contract=off",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall"]
 
-KERNEL_SOURCES = ["kernels/add_rmsnorm_quant.hip", "kernels/rope_rms.hip", "kernels/capi.cpp"]
+KERNEL_SOURCES = ["kernels/add_rmsnorm_quant.hip", "kernels/rope_rms.hip", "kernels/calibration.hip", "kernels/capi.cpp"]
 OP_SOURCES = ["register.cpp", "ops/allreduce_rms.cpp", "ops/fused_rope.cpp"]
 
 

@@ -43,18 +43,22 @@ __device__ __forceinline__ bool scale_in_fast_range(float s) {
     return s >= 0x1p-60f && s <= 0x1p60f;
 }
 
-template <typename T, int NCHUNK, int QUANT>
+// PAIRED: lanes 2k and 2k+1 swap half of their codes so that every lane issues one 16-byte store per two
+// chunks instead of two 8-byte stores (needs NCHUNK even and an even number of chunks per row).
+template <typename T, int NCHUNK, int QUANT, bool PAIRED>
 __global__ void __launch_bounds__(kMaxThreads)
 add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ residual_in,
                        const u32x4 *__restrict__ gamma, u32x4 *__restrict__ residual_out,
                        void *__restrict__ norm_out, float *__restrict__ scale_io, int chunks_per_row,
                        float hidden_f, float eps, float fp8_max) {
     using P = Pack16<T>;
+    static_assert(!PAIRED || NCHUNK % 2 == 0, "paired code stores need an even chunk count per lane");
     __shared__ float s_sum[kMaxWaves];
     __shared__ float s_max[kMaxWaves];
 
     const int tid = threadIdx.x;
-    const int num_waves = blockDim.x >> 6;
+    const int nthreads = blockDim.x;
+    const int num_waves = nthreads >> 6;
     const int64_t row_base = (int64_t)blockIdx.x * chunks_per_row;
 
     // ---- phase 0: issue every load of the row before touching any of them
@@ -62,7 +66,7 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
     bool live[NCHUNK];
 #pragma unroll
     for (int i = 0; i < NCHUNK; ++i) {
-        const int c = i * blockDim.x + tid;
+        const int c = i * nthreads + tid;
         live[i] = c < chunks_per_row;
         if (live[i]) {
             xv[i] = load_stream(x + row_base + c);
@@ -74,7 +78,7 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
     }
 #pragma unroll
     for (int i = 0; i < NCHUNK; ++i) {
-        const int c = i * blockDim.x + tid;
+        const int c = i * nthreads + tid;
         gv[i] = live[i] ? gamma[c] : u32x4{0, 0, 0, 0};
     }
 
@@ -86,17 +90,16 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
         for (int j = 0; j < 4; ++j) {
             const uint32_t w = P::pack(P::lo(xv[i][j]) + P::lo(rv[i][j]), P::hi(xv[i][j]) + P::hi(rv[i][j]));
             xv[i][j] = w;  // xv now holds the residual
-            const float a = P::lo(w), b = P::hi(w);
-            ss0 = __builtin_fmaf(a, a, ss0);
-            ss1 = __builtin_fmaf(b, b, ss1);
+            if (j & 1) ss1 = P::add_squares(w, ss1);
+            else ss0 = P::add_squares(w, ss0);
         }
-        if (live[i]) store_stream(residual_out + row_base + i * blockDim.x + tid, xv[i]);
+        if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
     }
     const float sumsq = block_allreduce<SumOp>(ss0 + ss1, s_sum, num_waves);
     const float rstd = 1.0f / sqrtf(sumsq / hidden_f + eps);
 
     // ---- phase 2: n2 = rT(gamma * rT(res * rstd)); row amax for the dynamic scale
-    float amax = 0.f;
+    uint32_t amax_bits = 0;
 #pragma unroll
     for (int i = 0; i < NCHUNK; ++i) {
 #pragma unroll
@@ -104,10 +107,7 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
             const uint32_t n1 = P::pack(P::lo(xv[i][j]) * rstd, P::hi(xv[i][j]) * rstd);
             const uint32_t n2 = P::pack(P::lo(gv[i][j]) * P::lo(n1), P::hi(gv[i][j]) * P::hi(n1));
             xv[i][j] = n2;  // xv now holds the normed row
-            if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
-                amax = __builtin_fmaxf(amax, __builtin_fabsf(P::lo(n2)));
-                amax = __builtin_fmaxf(amax, __builtin_fabsf(P::hi(n2)));
-            }
+            if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) amax_bits = absmax_packed(amax_bits, n2);
         }
     }
 
@@ -115,34 +115,59 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
         u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base;
 #pragma unroll
         for (int i = 0; i < NCHUNK; ++i)
-            if (live[i]) store_stream(out + i * blockDim.x + tid, xv[i]);
+            if (live[i]) store_stream(out + i * nthreads + tid, xv[i]);
         return;
     } else {
         float scale;
         if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
-            amax = block_allreduce<MaxOp>(amax, s_max, num_waves);
+            const float amax = block_allreduce<MaxOp>(absmax_to_float<T>(amax_bits), s_max, num_waves);
             scale = amax == 0.f ? 1.f : amax / fp8_max;
             if (tid == 0) scale_io[blockIdx.x] = scale;
         } else {
             scale = scale_io[0];
         }
 
-        // ---- phase 3: code = e4m3fn(clamp(n2 / scale)); 8 codes (one 8-byte store) per chunk
-        u32x2 *out = reinterpret_cast<u32x2 *>(norm_out) + row_base;
-        if (scale_in_fast_range(scale)) {
+        // ---- phase 3: code = e4m3fn(clamp(n2 / scale)), 8 codes per chunk.  With the dynamic scale
+        // |n2 / scale| <= 448 * (1 + 2^-23), which the converter already rounds to 448: no clamp needed.
+        constexpr bool kClamp = QUANT != GPUK_QUANT_FP8_DYNAMIC;
+        uint8_t *out = reinterpret_cast<uint8_t *>(norm_out) + row_base * 8;
+        if (__builtin_expect(scale_in_fast_range(scale), 1)) {
             const float rcp = 1.0f / scale;
-#pragma unroll
-            for (int i = 0; i < NCHUNK; ++i) {
+            auto encode = [&](const u32x4 &v) {
                 float q[8];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    q[2 * j] = clamp_sym(div_by_rcp(P::lo(xv[i][j]), scale, rcp), fp8_max);
-                    q[2 * j + 1] = clamp_sym(div_by_rcp(P::hi(xv[i][j]), scale, rcp), fp8_max);
+                    q[2 * j] = div_by_rcp(P::lo(v[j]), scale, rcp);
+                    q[2 * j + 1] = div_by_rcp(P::hi(v[j]), scale, rcp);
+                    if constexpr (kClamp) {
+                        q[2 * j] = clamp_sym(q[2 * j], fp8_max);
+                        q[2 * j + 1] = clamp_sym(q[2 * j + 1], fp8_max);
+                    }
                 }
-                u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
-                if (live[i]) store_stream(out + i * blockDim.x + tid, codes);
+                return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+            };
+            if constexpr (PAIRED) {
+                const bool odd = tid & 1;
+#pragma unroll
+                for (int i = 0; i < NCHUNK; i += 2) {
+                    const u32x2 c0 = encode(xv[i]), c1 = encode(xv[i + 1]);
+                    // the even lane keeps iteration i and sends i+1; the odd lane the other way round
+                    const u32x2 keep = odd ? c1 : c0, send = odd ? c0 : c1;
+                    const u32x2 recv = {dpp_xor1_u32(send[0]), dpp_xor1_u32(send[1])};
+                    const u32x4 both = odd ? u32x4{recv[0], recv[1], keep[0], keep[1]}
+                                           : u32x4{keep[0], keep[1], recv[0], recv[1]};
+                    const int c = odd ? (i + 1) * nthreads + tid - 1 : i * nthreads + tid;  // first chunk of the pair
+                    if (c < chunks_per_row) store_stream(reinterpret_cast<u32x4 *>(out + (int64_t)c * 8), both);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NCHUNK; ++i) {
+                    const u32x2 codes = encode(xv[i]);
+                    if (live[i]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
+                }
             }
         } else {
+            // scale so small or large that its reciprocal leaves the normal range: plain IEEE division
 #pragma unroll 1
             for (int i = 0; i < NCHUNK; ++i) {
                 float q[8];
@@ -151,8 +176,8 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
                     q[2 * j] = clamp_sym(P::lo(xv[i][j]) / scale, fp8_max);
                     q[2 * j + 1] = clamp_sym(P::hi(xv[i][j]) / scale, fp8_max);
                 }
-                u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
-                if (live[i]) store_stream(out + i * blockDim.x + tid, codes);
+                const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                if (live[i]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
             }
         }
     }
@@ -234,34 +259,43 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
     }
 }
 
-int g_force_nchunk = 0;  // 0 = heuristic; set through gpuk_set_tuning for sweeps
+int g_force_nchunk = 0;   // 0 = heuristic; set through gpuk_set_tuning for sweeps
+int g_force_threads = 0;  // 0 = heuristic
+int g_paired = 1;         // 16-byte paired code stores where the shape allows
 
-// Chunks per lane.  Few rows (decode): spread a row over as many lanes as possible to shorten the
-// dependent chain.  Many rows: 4 chunks per lane keeps 8 independent 16-byte loads in flight per lane
-// with 256-lane workgroups at hidden 8192.
-int pick_nchunk(int64_t tokens, int chunks_per_row) {
+// Lanes per row and chunks per lane.  Measured on MI355X with the traffic pattern alone: 512-lane
+// workgroups with 2 chunks per lane stream best for rows of 4096..8192 elements; shorter rows use one
+// chunk per lane; few rows (decode) spread each row over as many lanes as possible to shorten the
+// dependent load -> reduce -> reduce -> store chain.
+void pick_shape(int64_t tokens, int chunks_per_row, int *threads, int *nchunk) {
     auto fits = [&](int n) { return (int64_t)n * kMaxThreads >= chunks_per_row; };
+    int n;
     if (g_force_nchunk) {
-        int n = g_force_nchunk;
-        while (n < 8 && !fits(n)) n *= 2;
-        return fits(n) ? n : 0;
-    }
-    int n = 1;
-    if (tokens > 256) {
-        if (chunks_per_row >= 1024) n = 4;
-        else if (chunks_per_row >= 256) n = 2;
-    } else if (tokens > 32) {
-        if (chunks_per_row >= 512) n = 2;
+        n = g_force_nchunk;
+    } else if (tokens <= 256) {
+        n = 1;
+    } else {
+        n = 1;
+        while (n < 8 && chunks_per_row > 512 * n) n *= 2;
     }
     while (n < 8 && !fits(n)) n *= 2;
-    return fits(n) ? n : 0;
+    if (!fits(n)) {
+        *nchunk = 0;
+        *threads = kMaxThreads;
+        return;
+    }
+    int t = round_up((chunks_per_row + n - 1) / n, 64);
+    if (g_force_threads && (int64_t)g_force_threads * n >= chunks_per_row) t = g_force_threads;
+    *nchunk = n;
+    *threads = t;
 }
 
 template <typename T, int QUANT>
 int launch(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
            float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream) {
     const int chunks = (int)(hidden / 8);
-    const int nchunk = pick_nchunk(tokens, chunks);
+    int threads, nchunk;
+    pick_shape(tokens, chunks, &threads, &nchunk);
     const dim3 grid((unsigned)tokens);
     auto xs = static_cast<const u32x4 *>(x);
     auto rs = static_cast<const u32x4 *>(residual_in);
@@ -272,17 +306,15 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
         add_rmsnorm_quant_long_rows<T, QUANT><<<grid, kMaxThreads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale, chunks, hf, eps, fp8_max);
         return hip_status(hipGetLastError());
     }
-    const int threads = round_up((chunks + nchunk - 1) / nchunk, 64);
-#define GPUK_LAUNCH_NQ(N)                                                                                      \
-    case N:                                                                                                    \
-        add_rmsnorm_quant_rows<T, N, QUANT><<<grid, threads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale,     \
-                                                                          chunks, hf, eps, fp8_max);           \
-        break;
+    const bool paired = g_paired && QUANT != GPUK_QUANT_NONE && nchunk % 2 == 0 && chunks % 2 == 0;
+#define GPUK_LAUNCH_NQ(N, PAIRED)                                                                              \
+    add_rmsnorm_quant_rows<T, N, QUANT, PAIRED><<<grid, threads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale, \
+                                                                              chunks, hf, eps, fp8_max)
     switch (nchunk) {
-        GPUK_LAUNCH_NQ(1)
-        GPUK_LAUNCH_NQ(2)
-        GPUK_LAUNCH_NQ(4)
-        GPUK_LAUNCH_NQ(8)
+        case 1: GPUK_LAUNCH_NQ(1, false); break;
+        case 2: if (paired) GPUK_LAUNCH_NQ(2, true); else GPUK_LAUNCH_NQ(2, false); break;
+        case 4: if (paired) GPUK_LAUNCH_NQ(4, true); else GPUK_LAUNCH_NQ(4, false); break;
+        case 8: if (paired) GPUK_LAUNCH_NQ(8, true); else GPUK_LAUNCH_NQ(8, false); break;
         default: return GPUK_ERR_INTERNAL;
     }
 #undef GPUK_LAUNCH_NQ
@@ -307,7 +339,11 @@ int launch_quant(int quant_mode, const void *x, const void *residual_in, const v
 
 }  // namespace
 
-void set_norm_quant_nchunk(int n) { g_force_nchunk = n; }
+void set_norm_quant_tuning(int key, int value) {
+    if (key == 0) g_force_nchunk = value;
+    if (key == 1) g_force_threads = value;
+    if (key == 2) g_paired = value;
+}
 
 }  // namespace gpuk
 

@@ -22,7 +22,16 @@ extern "C" int gpuk_set_tuning(const char *key, int value) {
     if (!key) return GPUK_ERR_INVALID_ARG;
     if (strcmp(key, "norm_quant_nchunk") == 0) {
         if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8) return GPUK_ERR_INVALID_ARG;
-        gpuk::set_norm_quant_nchunk(value);
+        gpuk::set_norm_quant_tuning(0, value);
+        return GPUK_OK;
+    }
+    if (strcmp(key, "norm_quant_threads") == 0) {
+        if (value < 0 || value > 1024 || value % 64) return GPUK_ERR_INVALID_ARG;
+        gpuk::set_norm_quant_tuning(1, value);
+        return GPUK_OK;
+    }
+    if (strcmp(key, "norm_quant_paired_stores") == 0) {
+        gpuk::set_norm_quant_tuning(2, value != 0);
         return GPUK_OK;
     }
     if (strcmp(key, "rope_block_threads") == 0) {

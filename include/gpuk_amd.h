@@ -91,7 +91,8 @@ int gpuk_add_rmsnorm_quant(const void *x, const void *residual_in, const void *g
  *   qw, kw     : [head_size] `dtype`
  *   cos_sin    : [max_positions, head_size] `dtype`; row p = cos(p*f_0..f_{D/2-1}) | sin(...)
  *   positions  : int64; element (axis a, token t) at positions[a*pos_stride_axis + t*pos_stride_token]
- *   n_axes     : 1 (RoPE) or 3 (mRoPE; mrope_section[3] sums to head_size/2)
+ *   n_axes     : 1 (RoPE) or 3 (mRoPE; mrope_section is a HOST pointer to 3 values that sum to
+ *                head_size/2; it is read during the call and may be NULL when n_axes == 1)
  *   interleaved: mRoPE frequency->axis map; 0 chunked, 1 interleaved (rope_rms_impl.h:120-153)
  *   head_size  : 64, 128 or 256 (rope_rms_impl.h:473)
  */
@@ -121,6 +122,14 @@ int gpuk_rope_rms_set_kv(const void *qkv, const void *qw, const void *kw, const 
                          int64_t head_size, int is_neox_style, const int64_t *mrope_section, int is_interleaved,
                          float eps, int dtype, void *q_out, void *k_cache, void *v_cache, const int64_t *kv_loc,
                          float k_scale, float v_scale, int kv_dtype, void *stream);
+
+/*
+ * Roofline calibration: dst[0..nbytes) = src[0..nbytes) with a plain streaming copy kernel (nbytes a
+ * multiple of 16, both pointers 16-byte aligned).  Moves exactly 2*nbytes of HBM traffic; used to measure
+ * the practical bandwidth ceiling and to scale the profiler's FETCH_SIZE / WRITE_SIZE readings.
+ * Counterpart of the reference's micro-benchmark test/cpp/global_memory_bandwidth.cpp:95-114.
+ */
+int gpuk_copy_bytes(void *dst, const void *src, int64_t nbytes, void *stream);
 
 /* Development knob for sweeps: key "norm_quant_nchunk" (0 = heuristic, else 1/2/4/8 chunks per lane),
  * "rope_heads_per_wave" ... Unknown keys return GPUK_ERR_INVALID_ARG.  Not part of the reference. */

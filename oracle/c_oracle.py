@@ -56,6 +56,8 @@ def lib():
         L.gpuk_oracle_rope_rms_2way.restype = C.c_int
         L.gpuk_oracle_rope_rms_2way.argtypes = (
             [C.c_void_p] * 10 + [C.c_int64] * 6 + [C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p])
+        L.gpuk_oracle_count_div_rcp_mismatch.restype = C.c_int64
+        L.gpuk_oracle_count_div_rcp_mismatch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
         _lib = L
     return _lib
 
@@ -118,3 +120,9 @@ def rope_rms_2way(q0, k0, q1, k1, wq0, wk0, wq1, wk1, cs0, cs1, B, T0, T1, Hq, H
                                          DT[q0.dtype], _p(out_q), _p(out_k))
     assert rc == 0, rc
     return out_q, out_k
+
+
+def count_div_rcp_mismatch(a: torch.Tensor, b: torch.Tensor) -> int:
+    """a, b: fp32 CPU tensors of equal length; see gpuk_oracle_count_div_rcp_mismatch."""
+    assert a.dtype == torch.float32 and b.dtype == torch.float32 and a.numel() == b.numel()
+    return lib().gpuk_oracle_count_div_rcp_mismatch(_p(a.contiguous()), _p(b.contiguous()), a.numel())

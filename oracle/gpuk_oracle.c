@@ -329,3 +329,19 @@ int gpuk_oracle_rope_rms_2way(const uint16_t *q0, const uint16_t *k0, const uint
     }
     return 0;
 }
+
+/* Model of the device's reciprocal-based quotient (one multiply, two fused multiply-adds with
+ * rcp = RN(1/b)) against the IEEE quotient a/b: returns how many of the n pairs differ.  Lets the CPU
+ * tests show that the shortcut the HIP kernels take is exact on the operand ranges they guard. */
+int64_t gpuk_oracle_count_div_rcp_mismatch(const float *a, const float *b, int64_t n) {
+    int64_t bad = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        float rcp = 1.0f / b[i];
+        float q = a[i] * rcp;
+        float e = fmaf(-q, b[i], a[i]);
+        float q1 = fmaf(e, rcp, q);
+        float want = a[i] / b[i];
+        if (f32_bits(q1) != f32_bits(want) && !(q1 != q1 && want != want)) ++bad;
+    }
+    return bad;
+}

@@ -1,0 +1,172 @@
+"""CPU-only checks of the boundary: the C-ABI library loads and exports every symbol its header declares,
+the torch library registers the reference's operator schemas, argument validation rejects what it must
+without touching a GPU, and the host-side byte accounting matches the published per-configuration figures."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "gpuk_amd.h")
+
+
+def declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(gpuk_[a-z0-9_]+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol():
+    from gpuk_amd import capi
+
+    names = declared_functions()
+    assert set(names) == set(capi.EXPORTS), (names, capi.EXPORTS)
+    lib = ctypes.CDLL(os.path.join(ROOT, "gpuk_amd", "lib", "libgpuk_amd.so"))
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert capi.lib().gpuk_abi_version() == 1
+    assert capi.lib().gpuk_status_string(0) == b"ok"
+    assert b"unsupported" in capi.lib().gpuk_status_string(2)
+
+
+def test_argument_validation_needs_no_gpu():
+    """Bad arguments are rejected before any launch (status codes, not exceptions or aborts)."""
+    from gpuk_amd import capi
+
+    L = capi.lib()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p = (p + 15) & ~15
+    f = L.gpuk_add_rmsnorm_quant
+    assert f(p, p, p, p, p, p, -1, 1024, 1e-6, 0, 1, 448.0, None) == 1      # negative tokens
+    assert f(p, p, p, p, p, p, 4, 1020, 1e-6, 0, 1, 448.0, None) == 2       # hidden % 8
+    assert f(p, p, p, p, p, p, 4, 1024, 1e-6, 7, 1, 448.0, None) == 2       # unknown dtype
+    assert f(p, p, p, p, p, p, 4, 1024, 1e-6, 0, 2, 448.0, None) == 2       # e4m3fnuz
+    assert f(p, p, p, p, p, p, 4, 1024, 1e-6, 0, 9, 448.0, None) == 2       # unknown quant
+    assert f(p, p, p, p, p, None, 4, 1024, 1e-6, 0, 1, 448.0, None) == 1    # dynamic quant needs scale
+    assert f(p + 2, p, p, p, p, p, 4, 1024, 1e-6, 0, 1, 448.0, None) == 3   # misaligned
+    assert f(p, p, p, p, p, p, 4, 1024, 1e-6, 0, 1, 0.0, None) == 1         # fp8_max must be positive
+    assert f(None, None, None, None, None, None, 0, 1024, 1e-6, 0, 1, 448.0, None) == 0   # empty batch is a no-op
+    sec = (ctypes.c_int64 * 3)(16, 16, 16)
+    r = L.gpuk_rope_rms
+    assert r(p, p, p, p, p, 0, 1, 3, 4, 2, 2, 2, 128, 1, sec, 0, 1e-6, 0, None) == 1     # sections sum to 48, not 64
+    assert r(p, p, p, p, p, 0, 1, 1, 4, 2, 2, 2, 96, 1, None, 0, 1e-6, 0, None) == 2     # head size
+    assert r(p, p, p, p, p, 0, 1, 2, 4, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, None) == 1    # n_axes
+    assert r(p, p, p, p, p, 0, 1, 3, 4, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, None) == 1    # mRoPE without sections
+    assert r(None, None, None, None, None, 0, 1, 1, 0, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, None) == 0   # no tokens
+    s = L.gpuk_rope_rms_set_kv
+    assert s(p, p, p, p, p, 0, 1, 1, 4, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, p, p, p, p, 1.0, 1.0, 5, None) == 2  # kv dtype
+    assert s(p, p, p, p, p, 0, 1, 1, 4, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, p, p, p, p, 0.0, 1.0, 1, None) == 1  # fp8 scale
+    assert s(p, p, p, p, p, 0, 1, 1, 4, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, None, p, p, p, 1.0, 1.0, 0, None) == 1
+    assert L.gpuk_copy_bytes(p, p, 24, None) == 1 and L.gpuk_copy_bytes(p, p, 0, None) == 0
+    assert L.gpuk_set_tuning(b"no_such_knob", 1) == 1 and L.gpuk_set_tuning(b"norm_quant_nchunk", 3) == 1
+    assert L.gpuk_set_tuning(b"norm_quant_nchunk", 0) == 0
+
+
+def test_torch_library_registers_reference_schemas():
+    import gpuk_amd as gpuk
+
+    def schema(name):
+        return str(getattr(torch.ops.gpuk, name).default._schema)
+
+    assert schema("allreduce_rms") == (
+        "gpuk::allreduce_rms(SymInt fptr, Tensor allreduce_in, Tensor residual_in, Tensor rms_gamma, "
+        "Tensor residual_out, Tensor norm_out, Tensor scale_out, float eps, SymInt quant_type) -> ()")
+    assert schema("fused_rope_rms") == (
+        "gpuk::fused_rope_rms(Tensor qkv, Tensor qw, Tensor kw, Tensor cos_sin, Tensor positions, SymInt num_tokens, "
+        "SymInt num_heads_q, SymInt num_heads_k, SymInt num_heads_v, SymInt head_size, bool is_neox_style, "
+        "float eps) -> ()")
+    assert "int[] mrope_section_, bool is_interleaved, float eps) -> ()" in schema("fused_mrope_3d_rms")
+    assert schema("fused_mrope_3d_rms_set_kv").endswith(
+        "float eps, Tensor q, Tensor k_cache, Tensor v_cache, Tensor kv_loc, float k_scale, float v_scale) -> ()")
+    for name in ("allreduce_rms", "fused_rope_rms", "fused_mrope_3d_rms", "fused_mrope_3d_rms_set_kv",
+                 "fused_rope_rms_set_kv", "set_fp8_max", "get_fp8_max"):
+        assert hasattr(gpuk, name)
+    assert gpuk.fp8 == torch.float8_e4m3fn and gpuk.fp8_max_val == 448 and gpuk.fp8_policy_id == 1
+
+
+def test_fp8_max_setter_round_trip():
+    import gpuk_amd as gpuk
+
+    assert gpuk.get_fp8_max() == 448.0
+    gpuk.set_fp8_max(240.0)
+    try:
+        assert gpuk.get_fp8_max() == 240.0
+        with pytest.raises(RuntimeError):
+            gpuk.set_fp8_max(0.0)
+        with pytest.raises(RuntimeError):
+            gpuk.set_fp8_max(1000.0)
+    finally:
+        gpuk.set_fp8_max(448.0)
+
+
+def test_ops_refuse_cpu_tensors():
+    """There is no CPU fallback: the compute ops exist for GPU tensors only."""
+    import gpuk_amd as gpuk
+
+    x = torch.zeros((2, 64), dtype=torch.bfloat16)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        gpuk.allreduce_rms(0, x, x, x[0], x.clone(), x.clone(), torch.zeros(2, 1), 1e-6, 0)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        gpuk.fused_rope_rms(torch.zeros((2, 3, 64), dtype=torch.bfloat16), x[0], x[0], torch.zeros((8, 64), dtype=torch.bfloat16),
+                            torch.zeros(2, dtype=torch.int64), 2, 1, 1, 1, 64, True, 1e-6)
+
+
+def test_algorithmic_byte_formulas():
+    """Compulsory traffic per call, as published for the five configurations."""
+    from gpuk_amd import workloads as W
+
+    assert W.norm_quant_bytes(8192, 8192, 1) == 469_811_200
+    assert W.norm_quant_bytes(128, 4096, 3) == 3_678_212
+    assert [W.norm_quant_bytes(t, 7168, 1) for t in W.DECODE_TOKENS] == [64_516, 415_776, 1_620_096, 6_437_376, 25_706_496]
+    assert W.rope_set_kv_bytes(4096, 32, 8, 8, 128, 1, 2) == 101_777_920
+    assert W.rope_set_kv_bytes(8192, 28, 4, 4, 128, 3, 2) == 153_354_752
+    assert W.rope_set_kv_bytes(1, 64, 8, 8, 128, 1, 1) == 39_696 and W.rope_set_kv_bytes(512, 64, 8, 8, 128, 1, 1) == 20_062_720
+    # in-place form: the reference's own formula (test/cpp/test_rope_rms.cpp:184-188) plus the position read
+    T, hq, hk, D = 513, 32, 32, 128
+    ref = T * (hq + hk) * D * 2 + 2 * D * 2 + T * D * 2 + T * (hq + hk) * D * 2
+    assert W.rope_inplace_bytes(T, hq, hk, D) == ref + 8 * T
+
+
+def test_workload_generators_are_deterministic_and_shaped():
+    from gpuk_amd import workloads as W
+
+    a, b = W.config1(), W.config1()
+    assert torch.equal(a.x, b.x) and a.x.shape == (128, 4096) and a.x.dtype == torch.bfloat16
+    c2 = W.config2(64, 512)
+    frac = (c2.x.abs() == 50).float().mean().item()
+    assert 0.005 < frac < 0.015
+    c3 = W.config3(256)
+    assert c3.qkv.shape == (256, 48, 128) and c3.kv_loc.unique().numel() == 256 and c3.num_slots == 65536
+    assert c3.cos_sin.shape == (32768, 128) and c3.cos_sin[0, :64].eq(1).all() and c3.cos_sin[0, 64:].eq(0).all()
+    c4 = W.config4(4096)
+    pos = c4.positions
+    assert pos.shape == (3, 4096) and (pos[:, :1024] == torch.arange(1024)).all()
+    img = pos[:, 1024:2048]
+    assert (img[0] == 1024).all() and img[1].max() == 1024 + 31 and img[2].max() == 1024 + 31
+    assert (pos[:, 2048] == 1024 + 32).all() and c4.mrope_section == [16, 24, 24]
+    c5 = W.config5_rope(8)
+    assert c5.kv_dtype == torch.float8_e4m3fn and c5.qkv.shape == (8, 80, 128)
+
+
+def test_dist_env_rejects_multi_gpu_groups(monkeypatch):
+    import torch.distributed as dist
+
+    import gpuk_amd as gpuk
+
+    monkeypatch.setattr(dist, "is_initialized", lambda: True)
+    monkeypatch.setattr(dist, "get_rank", lambda group=None: 0)
+    monkeypatch.setattr(dist, "get_world_size", lambda group=None: 2)
+    monkeypatch.setattr(torch.cuda, "current_device", lambda: 0)
+    with pytest.raises(NotImplementedError):
+        gpuk.GPUKDistEnv(device_id=0)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "single-GPU" in r.stderr
