@@ -97,13 +97,13 @@ struct MaxOp {
     static __device__ __forceinline__ float apply(float a, float b) { return __builtin_fmaxf(a, b); }
 };
 
-// All-reduce over aligned groups of LANES consecutive lanes (LANES in {4, 8, 16}): every lane
+// All-reduce over aligned groups of LANES consecutive lanes (LANES in {2, 4, 8, 16}): every lane
 // ends with its group's result.  One DPP row is 16 lanes, so these never leave the row.
 template <typename Op, int LANES>
 __device__ __forceinline__ float group_allreduce(float v) {
-    static_assert(LANES == 4 || LANES == 8 || LANES == 16, "group must fit in one DPP row");
+    static_assert(LANES == 2 || LANES == 4 || LANES == 8 || LANES == 16, "group must fit in one DPP row");
     v = Op::apply(v, dpp_f32<DPP_QUAD_XOR1>(v));
-    v = Op::apply(v, dpp_f32<DPP_QUAD_XOR2>(v));
+    if constexpr (LANES >= 4) v = Op::apply(v, dpp_f32<DPP_QUAD_XOR2>(v));
     if constexpr (LANES >= 8) v = Op::apply(v, dpp_f32<DPP_ROW_HALF_MIRROR>(v));
     if constexpr (LANES >= 16) v = Op::apply(v, dpp_f32<DPP_ROW_MIRROR>(v));
     return v;

@@ -146,6 +146,33 @@ def test_rope_set_kv_head_mixes(device, hq, hk, hv, fp8):
     check_set_kv(inp, run_set_kv(inp, device), f"[set_kv {hq},{hk},{hv}]")
 
 
+@pytest.mark.parametrize("chunks_per_lane,rounds_per_wave,threads", [(2, 1, 128), (2, 4, 256), (4, 1, 256), (4, 3, 512), (2, 64, 64)])
+def test_launch_shape_variants(device, chunks_per_lane, rounds_per_wave, threads):
+    """Every selectable work decomposition (chunks per lane, rounds per wave, workgroup size) gives the same
+    bits as the oracle; the defaults are only the fastest of them."""
+    from gpuk_amd import capi
+
+    print(f"case variants cpl={chunks_per_lane} rpw={rounds_per_wave} threads={threads}", flush=True)
+    capi.set_tuning("rope_chunks_per_lane", chunks_per_lane)
+    capi.set_tuning("rope_rounds_per_wave", rounds_per_wave)
+    capi.set_tuning("rope_block_threads", threads)
+    try:
+        for hs, neox, mrope, fp8, heads in ((128, True, False, False, (32, 8, 8)), (64, False, True, True, (20, 20, 20)),
+                                            (256, True, True, False, (9, 3, 3)), (128, False, False, True, (64, 8, 8))):
+            inp = make(45, heads[0], hs, neox, seed=hs + rounds_per_wave, mrope=mrope, interleaved=mrope, fp8=fp8,
+                       hk=heads[1], hv=heads[2])
+            check_set_kv(inp, run_set_kv(inp, device), f"[variant D={hs}]")
+            got = run_inplace(inp, device)
+            want = oracle_inplace(inp)
+            nqk = heads[0] + heads[1]
+            assert_rotated_close(got[:, :nqk], want[:, :nqk], "in place q,k")
+            assert_bits_equal(got[:, nqk:], want[:, nqk:], "in place v")
+    finally:
+        capi.set_tuning("rope_chunks_per_lane", 2)
+        capi.set_tuning("rope_rounds_per_wave", 0)
+        capi.set_tuning("rope_block_threads", 0)
+
+
 def test_config3_qwen3_like(device):
     inp = workloads.config3()
     check_set_kv(inp, run_set_kv(inp, device), "[C3]")
