@@ -261,7 +261,7 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
 
 int g_force_nchunk = 0;   // 0 = heuristic; set through gpuk_set_tuning for sweeps
 int g_force_threads = 0;  // 0 = heuristic
-int g_paired = 1;         // 16-byte paired code stores where the shape allows
+int g_paired = 0;         // 16-byte paired code stores (measured no faster than 8-byte stores; kept selectable)
 
 // Lanes per row and chunks per lane.  Measured on MI355X with the traffic pattern alone: 512-lane
 // workgroups with 2 chunks per lane stream best for rows of 4096..8192 elements; shorter rows use one

@@ -113,7 +113,7 @@ def test_launch_shape_variants(device, threads, nchunk, paired):
     finally:
         capi.set_tuning("norm_quant_nchunk", 0)
         capi.set_tuning("norm_quant_threads", 0)
-        capi.set_tuning("norm_quant_paired_stores", 1)
+        capi.set_tuning("norm_quant_paired_stores", 0)
 
 
 def test_config1_static_per_tensor(device):
