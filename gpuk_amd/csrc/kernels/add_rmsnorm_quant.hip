@@ -43,37 +43,49 @@ __device__ __forceinline__ bool scale_in_fast_range(float s) {
     return s >= 0x1p-60f && s <= 0x1p60f;
 }
 
-// PAIRED: lanes 2k and 2k+1 swap half of their codes so that every lane issues one 16-byte store per two
-// chunks instead of two 8-byte stores (needs NCHUNK even and an even number of chunks per row).
-template <typename T, int NCHUNK, int QUANT, bool PAIRED>
+// ROWS: token rows a workgroup handles side by side (their loads are all in flight together and their two
+// reductions share the barriers).  PAIRED: lanes 2k and 2k+1 swap half of their codes so that every lane issues one
+// 16-byte store per two chunks instead of two 8-byte stores (needs NCHUNK even and an even number of chunks per row).
+template <typename T, int NCHUNK, int QUANT, bool PAIRED, int ROWS>
 __global__ void __launch_bounds__(kMaxThreads)
 add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ residual_in,
                        const u32x4 *__restrict__ gamma, u32x4 *__restrict__ residual_out,
-                       void *__restrict__ norm_out, float *__restrict__ scale_io, int chunks_per_row,
-                       float hidden_f, float eps, float fp8_max) {
+                       void *__restrict__ norm_out, float *__restrict__ scale_io, int tokens, int chunks_per_row,
+                       float hidden_f, float rcp_hidden, float eps, float fp8_max) {
     using P = Pack16<T>;
     static_assert(!PAIRED || NCHUNK % 2 == 0, "paired code stores need an even chunk count per lane");
-    __shared__ float s_sum[kMaxWaves];
-    __shared__ float s_max[kMaxWaves];
+    __shared__ float s_sum[ROWS * kReduceSlots];
+    __shared__ float s_max[ROWS * kReduceSlots];
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int num_waves = nthreads >> 6;
-    const int64_t row_base = (int64_t)blockIdx.x * chunks_per_row;
+    const int row0 = blockIdx.x * ROWS;
 
-    // ---- phase 0: issue every load of the row before touching any of them
-    u32x4 xv[NCHUNK], rv[NCHUNK], gv[NCHUNK];
+    // ---- phase 0: issue every load of the rows before touching any of them.  A row past the end re-reads the
+    // last row (its results are never stored), so the loads need no row predicate.
+    u32x4 xv[ROWS][NCHUNK], rv[ROWS][NCHUNK], gv[NCHUNK];
     bool live[NCHUNK];
+    int64_t row_base[ROWS];
+    bool row_ok[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        row_ok[r] = row0 + r < tokens;
+        row_base[r] = (int64_t)min(row0 + r, tokens - 1) * chunks_per_row;
+    }
 #pragma unroll
     for (int i = 0; i < NCHUNK; ++i) {
         const int c = i * nthreads + tid;
         live[i] = c < chunks_per_row;
-        if (live[i]) {
-            xv[i] = load_stream(x + row_base + c);
-            rv[i] = load_stream(residual_in + row_base + c);
-        } else {
-            xv[i] = u32x4{0, 0, 0, 0};
-            rv[i] = u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            if (live[i]) {
+                xv[r][i] = load_stream(x + row_base[r] + c);
+                rv[r][i] = load_stream(residual_in + row_base[r] + c);
+            } else {
+                xv[r][i] = u32x4{0, 0, 0, 0};
+                rv[r][i] = u32x4{0, 0, 0, 0};
+            }
         }
     }
 #pragma unroll
@@ -83,101 +95,122 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
     }
 
     // ---- phase 1: res = rT(x + r), stored once; sum of squares of the *rounded* residual
-    float ss0 = 0.f, ss1 = 0.f;
+    float sumsq[ROWS];
 #pragma unroll
-    for (int i = 0; i < NCHUNK; ++i) {
+    for (int r = 0; r < ROWS; ++r) {
+        float ss0 = 0.f, ss1 = 0.f;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t w = P::pack(P::lo(xv[i][j]) + P::lo(rv[i][j]), P::hi(xv[i][j]) + P::hi(rv[i][j]));
-            xv[i][j] = w;  // xv now holds the residual
-            if (j & 1) ss1 = P::add_squares(w, ss1);
-            else ss0 = P::add_squares(w, ss0);
+        for (int i = 0; i < NCHUNK; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t w = P::pack(P::lo(xv[r][i][j]) + P::lo(rv[r][i][j]), P::hi(xv[r][i][j]) + P::hi(rv[r][i][j]));
+                xv[r][i][j] = w;  // xv now holds the residual
+                if (j & 1) ss1 = P::add_squares(w, ss1);
+                else ss0 = P::add_squares(w, ss0);
+            }
+            if (live[i] && row_ok[r]) store_stream(residual_out + row_base[r] + i * nthreads + tid, xv[r][i]);
         }
-        if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+        sumsq[r] = ss0 + ss1;
     }
-    const float sumsq = block_allreduce<SumOp>(ss0 + ss1, s_sum, num_waves);
-    const float rstd = 1.0f / sqrtf(sumsq / hidden_f + eps);
+    block_allreduce<SumOp, ROWS>(sumsq, s_sum, num_waves);
 
     // ---- phase 2: n2 = rT(gamma * rT(res * rstd)); row amax for the dynamic scale
-    uint32_t amax_bits = 0;
+    float amax[ROWS];
 #pragma unroll
-    for (int i = 0; i < NCHUNK; ++i) {
+    for (int r = 0; r < ROWS; ++r) {
+        // mean = sumsq / H as an exact IEEE quotient: by the reciprocal of H (computed on the host) while that is
+        // safe, by a division otherwise
+        const float mean = (sumsq[r] >= 0x1p-60f && sumsq[r] <= 0x1p100f) ? div_by_rcp(sumsq[r], hidden_f, rcp_hidden)
+                                                                         : sumsq[r] / hidden_f;
+        const float rstd = 1.0f / sqrtf(mean + eps);
+        uint32_t amax_bits = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t n1 = P::pack(P::lo(xv[i][j]) * rstd, P::hi(xv[i][j]) * rstd);
-            const uint32_t n2 = P::pack(P::lo(gv[i][j]) * P::lo(n1), P::hi(gv[i][j]) * P::hi(n1));
-            xv[i][j] = n2;  // xv now holds the normed row
-            if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) amax_bits = absmax_packed(amax_bits, n2);
+        for (int i = 0; i < NCHUNK; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t n1 = P::pack(P::lo(xv[r][i][j]) * rstd, P::hi(xv[r][i][j]) * rstd);
+                const uint32_t n2 = P::pack(P::lo(gv[i][j]) * P::lo(n1), P::hi(gv[i][j]) * P::hi(n1));
+                xv[r][i][j] = n2;  // xv now holds the normed row
+                if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) amax_bits = absmax_packed(amax_bits, n2);
+            }
         }
+        amax[r] = absmax_to_float<T>(amax_bits);
     }
 
     if constexpr (QUANT == GPUK_QUANT_NONE) {
-        u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base;
 #pragma unroll
-        for (int i = 0; i < NCHUNK; ++i)
-            if (live[i]) store_stream(out + i * nthreads + tid, xv[i]);
+        for (int r = 0; r < ROWS; ++r) {
+            u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base[r];
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i)
+                if (live[i] && row_ok[r]) store_stream(out + i * nthreads + tid, xv[r][i]);
+        }
         return;
     } else {
-        float scale;
-        if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
-            const float amax = block_allreduce<MaxOp>(absmax_to_float<T>(amax_bits), s_max, num_waves);
-            scale = amax == 0.f ? 1.f : amax / fp8_max;
-            if (tid == 0) scale_io[blockIdx.x] = scale;
-        } else {
-            scale = scale_io[0];
-        }
-
-        // ---- phase 3: code = e4m3fn(clamp(n2 / scale)), 8 codes per chunk.  With the dynamic scale
-        // |n2 / scale| <= 448 * (1 + 2^-23), which the converter already rounds to 448: no clamp needed.
-        constexpr bool kClamp = QUANT != GPUK_QUANT_FP8_DYNAMIC;
-        uint8_t *out = reinterpret_cast<uint8_t *>(norm_out) + row_base * 8;
-        if (__builtin_expect(scale_in_fast_range(scale), 1)) {
-            const float rcp = 1.0f / scale;
-            auto encode = [&](const u32x4 &v) {
-                float q[8];
+        if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) block_allreduce<MaxOp, ROWS>(amax, s_max, num_waves);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    q[2 * j] = div_by_rcp(P::lo(v[j]), scale, rcp);
-                    q[2 * j + 1] = div_by_rcp(P::hi(v[j]), scale, rcp);
-                    if constexpr (kClamp) {
-                        q[2 * j] = clamp_sym(q[2 * j], fp8_max);
-                        q[2 * j + 1] = clamp_sym(q[2 * j + 1], fp8_max);
+        for (int r = 0; r < ROWS; ++r) {
+            float scale;
+            if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
+                scale = amax[r] == 0.f ? 1.f : amax[r] / fp8_max;
+                if (tid == 0 && row_ok[r]) scale_io[row0 + r] = scale;
+            } else {
+                scale = scale_io[0];
+            }
+
+            // ---- phase 3: code = e4m3fn(clamp(n2 / scale)), 8 codes per chunk.  With the dynamic scale
+            // |n2 / scale| <= 448 * (1 + 2^-23), which the converter already rounds to 448: no clamp needed.
+            constexpr bool kClamp = QUANT != GPUK_QUANT_FP8_DYNAMIC;
+            uint8_t *out = reinterpret_cast<uint8_t *>(norm_out) + row_base[r] * 8;
+            if (__builtin_expect(scale_in_fast_range(scale), 1)) {
+                const float rcp = 1.0f / scale;
+                auto encode = [&](const u32x4 &v) {
+                    float q[8];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        q[2 * j] = div_by_rcp(P::lo(v[j]), scale, rcp);
+                        q[2 * j + 1] = div_by_rcp(P::hi(v[j]), scale, rcp);
+                        if constexpr (kClamp) {
+                            q[2 * j] = clamp_sym(q[2 * j], fp8_max);
+                            q[2 * j + 1] = clamp_sym(q[2 * j + 1], fp8_max);
+                        }
+                    }
+                    return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                };
+                if constexpr (PAIRED) {
+                    const bool odd = tid & 1;
+#pragma unroll
+                    for (int i = 0; i < NCHUNK; i += 2) {
+                        const u32x2 c0 = encode(xv[r][i]), c1 = encode(xv[r][i + 1]);
+                        // the even lane keeps iteration i and sends i+1; the odd lane the other way round
+                        const u32x2 keep = odd ? c1 : c0, send = odd ? c0 : c1;
+                        const u32x2 recv = {dpp_xor1_u32(send[0]), dpp_xor1_u32(send[1])};
+                        const u32x4 both = odd ? u32x4{recv[0], recv[1], keep[0], keep[1]}
+                                               : u32x4{keep[0], keep[1], recv[0], recv[1]};
+                        const int c = odd ? (i + 1) * nthreads + tid - 1 : i * nthreads + tid;  // first chunk of the pair
+                        if (c < chunks_per_row && row_ok[r]) store_stream(reinterpret_cast<u32x4 *>(out + (int64_t)c * 8), both);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NCHUNK; ++i) {
+                        const u32x2 codes = encode(xv[r][i]);
+                        if (live[i] && row_ok[r]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
                     }
                 }
-                return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
-            };
-            if constexpr (PAIRED) {
-                const bool odd = tid & 1;
-#pragma unroll
-                for (int i = 0; i < NCHUNK; i += 2) {
-                    const u32x2 c0 = encode(xv[i]), c1 = encode(xv[i + 1]);
-                    // the even lane keeps iteration i and sends i+1; the odd lane the other way round
-                    const u32x2 keep = odd ? c1 : c0, send = odd ? c0 : c1;
-                    const u32x2 recv = {dpp_xor1_u32(send[0]), dpp_xor1_u32(send[1])};
-                    const u32x4 both = odd ? u32x4{recv[0], recv[1], keep[0], keep[1]}
-                                           : u32x4{keep[0], keep[1], recv[0], recv[1]};
-                    const int c = odd ? (i + 1) * nthreads + tid - 1 : i * nthreads + tid;  // first chunk of the pair
-                    if (c < chunks_per_row) store_stream(reinterpret_cast<u32x4 *>(out + (int64_t)c * 8), both);
-                }
             } else {
+                // scale so small or large that its reciprocal leaves the normal range: plain IEEE division
+                // (unrolled like the fast path: a runtime index into the register arrays would move them to LDS)
 #pragma unroll
                 for (int i = 0; i < NCHUNK; ++i) {
-                    const u32x2 codes = encode(xv[i]);
-                    if (live[i]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
-                }
-            }
-        } else {
-            // scale so small or large that its reciprocal leaves the normal range: plain IEEE division
-#pragma unroll 1
-            for (int i = 0; i < NCHUNK; ++i) {
-                float q[8];
+                    float q[8];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    q[2 * j] = clamp_sym(P::lo(xv[i][j]) / scale, fp8_max);
-                    q[2 * j + 1] = clamp_sym(P::hi(xv[i][j]) / scale, fp8_max);
+                    for (int j = 0; j < 4; ++j) {
+                        q[2 * j] = clamp_sym(P::lo(xv[r][i][j]) / scale, fp8_max);
+                        q[2 * j + 1] = clamp_sym(P::hi(xv[r][i][j]) / scale, fp8_max);
+                    }
+                    const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                    if (live[i] && row_ok[r]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
                 }
-                const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
-                if (live[i]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
             }
         }
     }
@@ -192,8 +225,8 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
                             float *__restrict__ scale_io, int chunks_per_row, float hidden_f, float eps,
                             float fp8_max) {
     using P = Pack16<T>;
-    __shared__ float s_sum[kMaxWaves];
-    __shared__ float s_max[kMaxWaves];
+    __shared__ float s_sum[kReduceSlots];
+    __shared__ float s_max[kReduceSlots];
     const int tid = threadIdx.x;
     const int num_waves = blockDim.x >> 6;
     const int64_t row_base = (int64_t)blockIdx.x * chunks_per_row;
@@ -210,8 +243,9 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
         }
         residual_out[row_base + c] = xv;
     }
-    const float sumsq = block_allreduce<SumOp>(ss, s_sum, num_waves);
-    const float rstd = 1.0f / sqrtf(sumsq / hidden_f + eps);
+    float sumsq[1] = {ss};
+    block_allreduce<SumOp, 1>(sumsq, s_sum, num_waves);
+    const float rstd = 1.0f / sqrtf(sumsq[0] / hidden_f + eps);
 
     auto normed = [&](int c) {
         u32x4 v = residual_out[row_base + c];  // written by this lane above
@@ -239,8 +273,9 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
                     amax = __builtin_fmaxf(amax, __builtin_fabsf(P::hi(v[j])));
                 }
             }
-            amax = block_allreduce<MaxOp>(amax, s_max, num_waves);
-            scale = amax == 0.f ? 1.f : amax / fp8_max;
+            float am[1] = {amax};
+            block_allreduce<MaxOp, 1>(am, s_max, num_waves);
+            scale = am[0] == 0.f ? 1.f : am[0] / fp8_max;
             if (tid == 0) scale_io[blockIdx.x] = scale;
         } else {
             scale = scale_io[0];
@@ -261,6 +296,8 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
 
 int g_force_nchunk = 0;   // 0 = heuristic; set through gpuk_set_tuning for sweeps
 int g_force_threads = 0;  // 0 = heuristic
+int g_rows = 0;           // rows per workgroup: 0 = heuristic, 1 or 2
+int g_lds_pad = 0;        // unused dynamic LDS bytes per workgroup: caps the workgroups resident per CU
 int g_paired = 0;         // 16-byte paired code stores (measured no faster than 8-byte stores; kept selectable)
 
 // Lanes per row and chunks per lane.  Measured on MI355X with the traffic pattern alone: 512-lane
@@ -307,16 +344,24 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
         return hip_status(hipGetLastError());
     }
     const bool paired = g_paired && QUANT != GPUK_QUANT_NONE && nchunk % 2 == 0 && chunks % 2 == 0;
-#define GPUK_LAUNCH_NQ(N, PAIRED)                                                                              \
-    add_rmsnorm_quant_rows<T, N, QUANT, PAIRED><<<grid, threads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale, \
-                                                                              chunks, hf, eps, fp8_max)
+    // two rows per workgroup once there are enough rows to keep every CU busy with half as many workgroups
+    const int rows = g_rows ? g_rows : 1;  // two rows per workgroup measured slower at every shape tried
+    const dim3 grid2((unsigned)((tokens + rows - 1) / rows));
+    const float rcp_hidden = 1.0f / hf;
+    const int tok = (int)tokens;
+#define GPUK_LAUNCH_NQ(N, PAIRED, ROWS)                                                                       \
+    add_rmsnorm_quant_rows<T, N, QUANT, PAIRED, ROWS><<<grid2, threads, g_lds_pad, stream>>>(xs, rs, gs, ro, norm_out, scale, tok, \
+                                                                                    chunks, hf, rcp_hidden, eps, fp8_max)
+#define GPUK_LAUNCH_NQ_ROWS(N, PAIRED) \
+    if (rows == 2) GPUK_LAUNCH_NQ(N, PAIRED, 2); else GPUK_LAUNCH_NQ(N, PAIRED, 1)
     switch (nchunk) {
-        case 1: GPUK_LAUNCH_NQ(1, false); break;
-        case 2: if (paired) GPUK_LAUNCH_NQ(2, true); else GPUK_LAUNCH_NQ(2, false); break;
-        case 4: if (paired) GPUK_LAUNCH_NQ(4, true); else GPUK_LAUNCH_NQ(4, false); break;
-        case 8: if (paired) GPUK_LAUNCH_NQ(8, true); else GPUK_LAUNCH_NQ(8, false); break;
+        case 1: GPUK_LAUNCH_NQ_ROWS(1, false); break;
+        case 2: if (paired) { GPUK_LAUNCH_NQ_ROWS(2, true); } else { GPUK_LAUNCH_NQ_ROWS(2, false); } break;
+        case 4: if (paired) { GPUK_LAUNCH_NQ_ROWS(4, true); } else { GPUK_LAUNCH_NQ_ROWS(4, false); } break;
+        case 8: if (paired) GPUK_LAUNCH_NQ(8, true, 1); else GPUK_LAUNCH_NQ(8, false, 1); break;
         default: return GPUK_ERR_INTERNAL;
     }
+#undef GPUK_LAUNCH_NQ_ROWS
 #undef GPUK_LAUNCH_NQ
     return hip_status(hipGetLastError());
 }
@@ -343,6 +388,8 @@ void set_norm_quant_tuning(int key, int value) {
     if (key == 0) g_force_nchunk = value;
     if (key == 1) g_force_threads = value;
     if (key == 2) g_paired = value;
+    if (key == 3) g_rows = value;
+    if (key == 4) g_lds_pad = value;
 }
 
 }  // namespace gpuk

@@ -92,9 +92,11 @@ constexpr int DPP_ROW_MIRROR = 0x140;
 
 struct SumOp {
     static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
+    static __device__ __forceinline__ float identity() { return 0.f; }
 };
-struct MaxOp {
+struct MaxOp {  // used on magnitudes only, so 0 is the identity
     static __device__ __forceinline__ float apply(float a, float b) { return __builtin_fmaxf(a, b); }
+    static __device__ __forceinline__ float identity() { return 0.f; }
 };
 
 // All-reduce over aligned groups of LANES consecutive lanes (LANES in {2, 4, 8, 16}): every lane
@@ -122,19 +124,28 @@ __device__ __forceinline__ float wave_allreduce(float v) {
     return Op::apply(Op::apply(r0, r1), Op::apply(r2, r3));
 }
 
-// Workgroup all-reduce: wave results meet in LDS (one float per wave, at most 16 waves) and
-// every thread folds them in wave order.  `slots` must be private to this call site so that two
-// consecutive reductions need only one barrier each.
-template <typename Op>
-__device__ __forceinline__ float block_allreduce(float v, float *slots, int num_waves) {
-    v = wave_allreduce<Op>(v);
-    if (num_waves == 1) return v;
+// Workgroup all-reduce of N independent values: wave results meet in LDS (N x 16 floats, at most 16 waves), one
+// barrier, then every wave reads the per-wave results into its lanes (lane l takes wave l mod 16) and folds them with
+// four DPP steps, so the result is the same in every lane of the workgroup.  `slots` must be private to this call
+// site so that two consecutive reductions need only one barrier each.
+constexpr int kReduceSlots = 16;
+template <typename Op, int N>
+__device__ __forceinline__ void block_allreduce(float (&v)[N], float *slots, int num_waves) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) v[n] = wave_allreduce<Op>(v[n]);
+    if (num_waves == 1) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (lane == 0) slots[wave] = v;
+    if (lane == 0) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) slots[n * kReduceSlots + wave] = v[n];
+    }
     __syncthreads();
-    float acc = slots[0];
-    for (int w = 1; w < num_waves; ++w) acc = Op::apply(acc, slots[w]);
-    return acc;
+    const int src = lane & (kReduceSlots - 1);
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+        const float s = slots[n * kReduceSlots + src];
+        v[n] = group_allreduce<Op, 16>(src < num_waves ? s : Op::identity());
+    }
 }
 
 // Four fp32 -> four OCP e4m3fn codes in one dword (two v_cvt_pk_fp8_f32).  Inputs must already be

@@ -94,19 +94,21 @@ def test_every_chunking_variant(device, nchunk):
         capi.set_tuning("norm_quant_nchunk", 0)
 
 
-@pytest.mark.parametrize("threads,nchunk,paired", [(512, 2, 1), (512, 2, 0), (256, 4, 1), (1024, 2, 1), (128, 8, 1), (448, 2, 1)])
-def test_launch_shape_variants(device, threads, nchunk, paired):
-    """Workgroup size, chunks per lane and the paired 16-byte code stores are tuning choices only."""
+@pytest.mark.parametrize("threads,nchunk,paired,rows", [(512, 2, 1, 1), (512, 2, 0, 2), (256, 4, 1, 2), (1024, 2, 1, 1),
+                                                        (128, 8, 1, 1), (448, 2, 1, 2), (1024, 1, 0, 2), (256, 4, 0, 1)])
+def test_launch_shape_variants(device, threads, nchunk, paired, rows):
+    """Workgroup size, chunks per lane, rows per workgroup and the paired 16-byte code stores are tuning choices only."""
     from gpuk_amd import capi
 
-    print(f"case variants threads={threads} nchunk={nchunk} paired={paired}", flush=True)
+    print(f"case variants threads={threads} nchunk={nchunk} paired={paired} rows={rows}", flush=True)
     capi.set_tuning("norm_quant_nchunk", nchunk)
     capi.set_tuning("norm_quant_threads", threads)
     capi.set_tuning("norm_quant_paired_stores", paired)
+    capi.set_tuning("norm_quant_rows", rows)
     try:
         for hidden in (8192, 7168, 1032):
-            inp = workloads.norm_quant_inputs(300, hidden, seed=threads + hidden, res_sigma=2.0, outlier_frac=0.01)
-            for quant in (1, 3):
+            inp = workloads.norm_quant_inputs(301, hidden, seed=threads + hidden, res_sigma=2.0, outlier_frac=0.01)
+            for quant in (0, 1, 3):
                 st = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
                 check(inp, quant, run_capi(inp, quant, device, static_scale=st), static_scale=st,
                       tag=f"[variant H={hidden} q{quant}]")
@@ -114,6 +116,7 @@ def test_launch_shape_variants(device, threads, nchunk, paired):
         capi.set_tuning("norm_quant_nchunk", 0)
         capi.set_tuning("norm_quant_threads", 0)
         capi.set_tuning("norm_quant_paired_stores", 0)
+        capi.set_tuning("norm_quant_rows", 0)
 
 
 def test_config1_static_per_tensor(device):
