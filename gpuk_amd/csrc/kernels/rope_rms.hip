@@ -4,12 +4,15 @@
 // Stands behind the reference's fused_rope_rms, fused_mrope_3d_rms and fused_mrope_3d_rms_set_kv
 // (host ops src/ops/fused_rope.cpp:19-166, kernels src/impl/rope_rms_impl.h:157-466, launchers :468-610).
 // The reference maps one 32-lane group to one head with D/32 elements per lane, fetches the rotation
-// partner with two vector shuffles and re-gathers cos/sin element by element for every head.  Here a head
-// is D/32 lanes of a wave64 and every lane owns four 16-byte chunks (32 elements) that already contain
-// both members of each rotation pair, so the rotation needs no cross-lane traffic, the sum of squares is
-// reduced inside one DPP quad or row, and the per-head scalar work (rstd) is shared by twice as many
-// elements.  A wave covers 64/(D/32) heads per round and loops over rounds of the same token and kind,
-// so the position lookup, the mRoPE axis selection and the cos/sin and weight loads happen once per wave.
+// partner with two vector shuffles and gathers cos/sin element by element, per head, with 64-bit modulo
+// arithmetic.  Here a head is D/16 lanes of a wave64 and every lane owns two 16-byte chunks that already
+// contain both members of each rotation pair, so the rotation needs no cross-lane traffic and the sum of
+// squares is reduced with 2-4 DPP steps inside one 16-lane row.
+//
+// Work decomposition: Q and K heads of a token form one index space of Hq+Hk heads; one wave takes 64/(D/16)
+// consecutive heads of one token (2 KiB of contiguous qkv at D=128), whether they are Q, K or a mix (the norm
+// weights and the destination are chosen per lane).  With a KV cache, the waves of a token also share out the
+// token's V row, one 16-byte chunk per lane, so no wave exists only to copy.
 //
 // Numerics follow the reference's torch oracle (test/test_fused_rope_rms.py:8-34,
 // test/test_fused_mrope_rms_set_kv.py:62-130), rT = round-to-nearest-even into the 16-bit type:
@@ -39,8 +42,10 @@ struct RopeArgs {
     int64_t ps_axis, ps_token;
     void *q_out, *k_cache, *v_cache;
     const int64_t *kv_loc;
-    // work decomposition: a unit is (token, kind q|k|v, block of `rounds_per_wave` rounds); one wave per unit
-    uint32_t total_units, units_per_token, units_q, units_k, rounds_per_wave;
+    // one wave per unit = (token, group of heads); units_per_token = ceil((hq + hk) / heads per wave)
+    uint32_t total_units, units_per_token;
+    uint32_t upt_magic;  // ceil(2^32 / units_per_token), or 0 when units_per_token is 1: unit / units_per_token is
+                         // mulhi(unit, magic) for every unit the host admits
     int hq, hk, hv;
     float eps, k_scale, v_scale;
     // mRoPE: bit f of axis1 / axis2 set when rotary frequency f takes its position from axis 1 / 2
@@ -60,315 +65,239 @@ __device__ __forceinline__ float elem(const u32x4 &v, int e) {  // element e (0.
     return (e & 1) ? Pack16<T>::hi(v[e >> 1]) : Pack16<T>::lo(v[e >> 1]);
 }
 
-// Divides by a scale that is the same for the whole launch; `rcp` is RN(1/scale) when `fast`.
-struct Divider {
-    float scale, rcp;
-    bool fast;
-    __device__ __forceinline__ explicit Divider(float s)
-        : scale(s), rcp(1.0f / s), fast(s >= 0x1p-60f && s <= 0x1p60f) {}
-    __device__ __forceinline__ float operator()(float a) const {
-        return fast ? div_by_rcp(a, scale, rcp) : a / scale;
-    }
-};
-
-// 8 codes = e4m3fn(clamp(rT(v / scale))) for one chunk
+// 8 codes = e4m3fn(clamp(rT(v / scale))) for one chunk; `rcp` is RN(1/scale) and is used when FAST
 template <typename T, bool FAST>
-__device__ __forceinline__ u32x2 quantize_chunk(const u32x4 &v, const Divider &d) {
+__device__ __forceinline__ u32x2 quantize_chunk(const u32x4 &v, float scale, float rcp) {
     using P = Pack16<T>;
     float q[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const float a = FAST ? div_by_rcp(P::lo(v[j]), d.scale, d.rcp) : P::lo(v[j]) / d.scale;
-        const float b = FAST ? div_by_rcp(P::hi(v[j]), d.scale, d.rcp) : P::hi(v[j]) / d.scale;
+        const float a = FAST ? div_by_rcp(P::lo(v[j]), scale, rcp) : P::lo(v[j]) / scale;
+        const float b = FAST ? div_by_rcp(P::hi(v[j]), scale, rcp) : P::hi(v[j]) / scale;
         const uint32_t w = P::pack(a, b);
         q[2 * j] = clamp_sym(P::lo(w), kE4M3Max);
         q[2 * j + 1] = clamp_sym(P::hi(w), kE4M3Max);
     }
     return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
 }
+__device__ __forceinline__ bool scale_is_fast(float s) { return s >= 0x1p-60f && s <= 0x1p60f; }
 
-// Chunk ids (units of 8 elements inside a head) owned by lane `sub` of the head's LPH = D/(8*CPL) lanes, for
-// CPL = 2 or 4 chunks per lane.  HC = chunks per half head.
-//   NeoX  : the first CPL/2 slots come from the first half of the head, slot i + CPL/2 is the chunk D/2 elements
-//           further, so slot i pairs with slot i + CPL/2 under table chunk i.
-//   GPT-J : runs of two adjacent chunks {2sub, 2sub+1} (and {2sub+HC, 2sub+1+HC} for CPL 4); pairs sit inside a
-//           chunk, and a run of two chunks uses one table chunk.
-// In both styles the lane's rotary frequencies are the table chunks {sub} (CPL 2) or {sub, sub+LPH} (CPL 4) of
-// the cos half and of the sin half.
-template <int D, bool NEOX, int CPL>
-__device__ __forceinline__ void chunk_ids(int sub, int (&c)[CPL]) {
-    constexpr int HC = D / 16, LPH = D / (8 * CPL);
-    if constexpr (NEOX) {
-#pragma unroll
-        for (int i = 0; i < CPL / 2; ++i) {
-            c[i] = sub + i * LPH;
-            c[i + CPL / 2] = HC + sub + i * LPH;
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < CPL / 2; ++i) {
-            c[2 * i] = 2 * sub + i * HC;
-            c[2 * i + 1] = 2 * sub + 1 + i * HC;
-        }
-    }
-}
-
-// Keeps the compiler from hoisting the unpacking of a loop-invariant packed dword out of the round loop
-// (the unpacked copies would double the register count and halve the occupancy).
-__device__ __forceinline__ uint32_t opaque(uint32_t v) {
-    asm volatile("" : "+v"(v));
-    return v;
-}
+// What one wave keeps about one unit (= one group of 64/(D/16) consecutive Q/K heads of one token, plus its share
+// of the token's V row) between issuing the unit's loads and finishing it.
+struct UnitState {
+    uint32_t t, u;
+    int head;
+    bool live, active, is_q;
+    int64_t slot;
+    const uint16_t *token_in;
+    u32x4 xa, xb, wa, wb, cosv, sinv, vchunk;
+};
 
 // AXES: 1 = RoPE, 3 = mRoPE.  SETKV: false = in place, true = scatter to q_out / caches.
-// CPL: 16-byte chunks per lane and head (2 or 4).
-template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8, int CPL>
-__global__ void __launch_bounds__(512) rope_rms_kernel(const RopeArgs a) {
+template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
+struct RopeUnit {
     using P = Pack16<T>;
-    constexpr int LPH = D / (8 * CPL);  // lanes per head
-    constexpr int HPW = 64 / LPH;       // heads per wave and round
-    constexpr int HALF = D / 2;
-    constexpr int NT = CPL / 2;         // table chunks (of cos and of sin) per lane
+    static constexpr int LPH = D / 16;    // lanes per head
+    static constexpr int HPW = 64 / LPH;  // heads per wave
+    static constexpr int HALF = D / 2;
 
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t unit = blockIdx.x * (blockDim.x >> 6) + wave;
-    if (unit >= a.total_units) return;
-    const uint32_t t = unit / a.units_per_token;
-    const uint32_t u = unit - t * a.units_per_token;
+    // element offsets of a lane's two chunks inside a head (NeoX: x1 chunk and the chunk D/2 further; GPT-J: two
+    // adjacent chunks) and of its cos / sin chunks inside a table row
+    static __device__ __forceinline__ int c0(int sub) { return NEOX ? 8 * sub : 16 * sub; }
+    static __device__ __forceinline__ int c1(int sub) { return NEOX ? HALF + 8 * sub : 16 * sub + 8; }
 
-    const int lane = threadIdx.x & 63;
-    const int sub = lane % LPH;
-    const int hl = lane / LPH;
-    const int heads_all = a.hq + a.hk + a.hv;
-    const uint16_t *token_in = static_cast<const uint16_t *>(a.qkv_in) + (int64_t)t * heads_all * D;
+    // Issues every load of the unit; nothing is waited for.
+    static __device__ __forceinline__ void issue_loads(const RopeArgs &a, uint32_t unit, int lane, UnitState &st) {
+        st.live = unit < a.total_units;  // wave-uniform
+        if (!st.live) return;
+        st.t = a.upt_magic ? __umulhi(unit, a.upt_magic) : unit;
+        st.u = unit - st.t * a.units_per_token;
+        const int sub = lane % LPH, hl = lane / LPH;
+        const int heads_qk = a.hq + a.hk, heads_all = heads_qk + a.hv;
+        st.token_in = static_cast<const uint16_t *>(a.qkv_in) + (int64_t)st.t * heads_all * D;
 
-    if (u < a.units_q + a.units_k) {
-        // ------------------------------------------------------------------ Q or K heads
-        const bool is_q = u < a.units_q;
-        const int heads_kind = is_q ? a.hq : a.hk;
-        const int head_base = is_q ? 0 : a.hq;  // first head of this kind inside the token
-        const int round0 = (is_q ? u : u - a.units_q) * a.rounds_per_wave;
-        const int rounds_kind = (heads_kind + HPW - 1) / HPW;
-        const int round1 = min(round0 + (int)a.rounds_per_wave, rounds_kind);
+        // lanes past the last head re-read the last head (nothing of theirs is stored): no branch around the loads
+        const int head_raw = st.u * HPW + hl;
+        st.active = head_raw < heads_qk;
+        st.head = min(head_raw, heads_qk - 1);
+        st.is_q = st.head < a.hq;
+        const uint16_t *src = st.token_in + (int64_t)st.head * D;
+        st.xa = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c0(sub)));
+        st.xb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c1(sub)));
 
-        int cid[CPL];
-        chunk_ids<D, NEOX, CPL>(sub, cid);
-        // Lanes past the last head of the kind re-read the last head (their results are never stored): the load
-        // needs no branch, which keeps the compiler's wait counters exact inside the round loop.
-        auto load_head = [&](int round, u32x4(&x)[CPL]) {
-            const int head = min(round * HPW + hl, heads_kind - 1);
-            const uint16_t *src = token_in + (int64_t)(head_base + head) * D;
-#pragma unroll
-            for (int i = 0; i < CPL; ++i) x[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 8 * cid[i]));
-        };
-        u32x4 cur[CPL], nxt[CPL];
-        load_head(round0, cur);
-
-        // per-wave constants: norm weights of the lane's chunks, cos / sin of the lane's frequencies
-        const uint16_t *wsrc = static_cast<const uint16_t *>(is_q ? a.qw : a.kw);
-        u32x4 w[CPL];
-#pragma unroll
-        for (int i = 0; i < CPL; ++i) w[i] = *reinterpret_cast<const u32x4 *>(wsrc + 8 * cid[i]);
-
-        const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin);
-        const int64_t p0 = a.positions[(int64_t)t * a.ps_token];
-        u32x4 cosv[NT], sinv[NT];
-#pragma unroll
-        for (int k = 0; k < NT; ++k) {
-            const int f = 8 * (sub + k * LPH);  // first frequency of the lane's table chunk k
-            cosv[k] = *reinterpret_cast<const u32x4 *>(table + p0 * D + f);
-            sinv[k] = *reinterpret_cast<const u32x4 *>(table + p0 * D + HALF + f);
-        }
-        if constexpr (AXES == 3) {
-            const int64_t p1 = a.positions[a.ps_axis + (int64_t)t * a.ps_token];
-            const int64_t p2 = a.positions[2 * a.ps_axis + (int64_t)t * a.ps_token];
-            if (p1 != p0 || p2 != p0) {  // wave-uniform; text tokens carry three equal positions
-#pragma unroll
-                for (int k = 0; k < NT; ++k) {
-                    const int f = 8 * (sub + k * LPH);
-                    const u32x4 cos1 = *reinterpret_cast<const u32x4 *>(table + p1 * D + f);
-                    const u32x4 sin1 = *reinterpret_cast<const u32x4 *>(table + p1 * D + HALF + f);
-                    const u32x4 cos2 = *reinterpret_cast<const u32x4 *>(table + p2 * D + f);
-                    const u32x4 sin2 = *reinterpret_cast<const u32x4 *>(table + p2 * D + HALF + f);
-                    // 8 axis bits for frequencies f .. f+7 (f is a multiple of 8, so they share a word)
-                    const uint32_t b1 = (a.axis1[f >> 5] >> (f & 31)) & 0xffu;
-                    const uint32_t b2 = (a.axis2[f >> 5] >> (f & 31)) & 0xffu;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint32_t m1 = halves_mask(b1 >> (2 * j)), m2 = halves_mask(b2 >> (2 * j));
-                        cosv[k][j] = bitselect(m2, cos2[j], bitselect(m1, cos1[j], cosv[k][j]));
-                        sinv[k][j] = bitselect(m2, sin2[j], bitselect(m1, sin1[j], sinv[k][j]));
-                    }
-                }
-            }
-        }
-
-        int64_t slot = 0;
+        // this wave's share of the token's V row: chunk u*64 + lane (and further strides of units_per_token*64)
         if constexpr (SETKV) {
-            if (!is_q) slot = a.kv_loc[t];
+            st.slot = a.kv_loc[st.t];
+            const int v_first = st.u * 64 + lane;
+            if (v_first < a.hv * (D / 8))
+                st.vchunk = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(st.token_in + (int64_t)heads_qk * D + 8 * v_first));
         }
-        const Divider kdiv(a.k_scale);
-        // row of head 0 of this kind in the 16-bit destination (in place / q_out / k_cache slot)
-        uint16_t *out_row;
-        if constexpr (!SETKV) out_row = static_cast<uint16_t *>(a.qkv_out) + ((int64_t)t * heads_all + head_base) * D;
-        else out_row = is_q ? static_cast<uint16_t *>(a.q_out) + (int64_t)t * a.hq * D
-                            : static_cast<uint16_t *>(a.k_cache) + slot * a.hk * D;
 
-        // All set-up loads (weights, cos/sin, first round) have to land before the loop: the waits the compiler
-        // would otherwise place inside it also cover the prefetch of the next round and serialise the rounds.
-        if (round1 - round0 > 1) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-#pragma unroll 1
-        for (int round = round0; round < round1; ++round) {
-            if (round + 1 < round1) load_head(round + 1, nxt);
+        const uint16_t *wsrc = static_cast<const uint16_t *>(st.is_q ? a.qw : a.kw);
+        st.wa = *reinterpret_cast<const u32x4 *>(wsrc + c0(sub));
+        st.wb = *reinterpret_cast<const u32x4 *>(wsrc + c1(sub));
 
-            // RMSNorm over the head: LPH lanes x 8*CPL elements
-            float ss0 = 0.f, ss1 = 0.f;
-#pragma unroll
-            for (int i = 0; i < CPL; ++i) {
-                ss0 = P::add_squares(cur[i][0], ss0);
-                ss1 = P::add_squares(cur[i][1], ss1);
-                ss0 = P::add_squares(cur[i][2], ss0);
-                ss1 = P::add_squares(cur[i][3], ss1);
-            }
-            const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
-            const float rstd = 1.0f / sqrtf(sumsq * (1.0f / D) + a.eps);  // D is a power of two: exact
-
-            u32x4 n[CPL];
-#pragma unroll
-            for (int i = 0; i < CPL; ++i) {
+        const int fc = 8 * sub;
+        const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin);
+        const int64_t p0 = a.positions[(int64_t)st.t * a.ps_token];
+        st.cosv = *reinterpret_cast<const u32x4 *>(table + p0 * D + fc);
+        st.sinv = *reinterpret_cast<const u32x4 *>(table + p0 * D + HALF + fc);
+        if constexpr (AXES == 3) {
+            const int64_t p1 = a.positions[a.ps_axis + (int64_t)st.t * a.ps_token];
+            const int64_t p2 = a.positions[2 * a.ps_axis + (int64_t)st.t * a.ps_token];
+            if (p1 != p0 || p2 != p0) {  // wave-uniform; text tokens carry three equal positions
+                const u32x4 cos1 = *reinterpret_cast<const u32x4 *>(table + p1 * D + fc);
+                const u32x4 sin1 = *reinterpret_cast<const u32x4 *>(table + p1 * D + HALF + fc);
+                const u32x4 cos2 = *reinterpret_cast<const u32x4 *>(table + p2 * D + fc);
+                const u32x4 sin2 = *reinterpret_cast<const u32x4 *>(table + p2 * D + HALF + fc);
+                // 8 axis bits for frequencies fc .. fc+7 (fc is a multiple of 8, so they share a word)
+                const uint32_t b1 = (a.axis1[fc >> 5] >> (fc & 31)) & 0xffu;
+                const uint32_t b2 = (a.axis2[fc >> 5] >> (fc & 31)) & 0xffu;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const uint32_t wj = opaque(w[i][j]);
-                    const uint32_t s = P::pack(P::lo(cur[i][j]) * rstd, P::hi(cur[i][j]) * rstd);
-                    n[i][j] = P::pack(P::lo(wj) * P::lo(s), P::hi(wj) * P::hi(s));
-                }
-            }
-
-            u32x4 o[CPL];
-            if constexpr (NEOX) {
-                // slot i holds x1 and slot i + CPL/2 the matching x2 for the 8 frequencies of table chunk i
-#pragma unroll
-                for (int i = 0; i < NT; ++i) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint32_t cj = opaque(cosv[i][j]), sj = opaque(sinv[i][j]);
-                        const float x1l = P::lo(n[i][j]), x1h = P::hi(n[i][j]);
-                        const float x2l = P::lo(n[i + NT][j]), x2h = P::hi(n[i + NT][j]);
-                        const float cl = P::lo(cj), ch = P::hi(cj), sl = P::lo(sj), sh = P::hi(sj);
-                        const uint32_t t1 = P::pack(x1l * cl, x1h * ch), t2 = P::pack(x2l * sl, x2h * sh);
-                        const uint32_t t3 = P::pack(x2l * cl, x2h * ch), t4 = P::pack(x1l * sl, x1h * sh);
-                        o[i][j] = P::pack(P::lo(t1) - P::lo(t2), P::hi(t1) - P::hi(t2));
-                        o[i + NT][j] = P::pack(P::lo(t3) + P::lo(t4), P::hi(t3) + P::hi(t4));
-                    }
-                }
-            } else {
-                // each dword is one (x1, x2) pair; slots 2k, 2k+1 use elements 0-3 and 4-7 of table chunk k
-#pragma unroll
-                for (int i = 0; i < CPL; ++i) {
-                    u32x4 ck, sk;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        ck[j] = opaque(cosv[i >> 1][j]);
-                        sk[j] = opaque(sinv[i >> 1][j]);
-                    }
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float x1 = P::lo(n[i][e]), x2 = P::hi(n[i][e]);
-                        const float c = elem<T>(ck, 4 * (i & 1) + e), s = elem<T>(sk, 4 * (i & 1) + e);
-                        const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
-                        o[i][e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
-                    }
-                }
-            }
-
-            // The prefetch has had the whole round to land.  Waiting for it here, while it is the youngest
-            // outstanding access, keeps this round's stores out of the wait.
-            if (round + 1 < round1) {
-                __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-#pragma unroll
-                for (int i = 0; i < CPL; ++i) cur[i] = nxt[i];
-            }
-            const int head = round * HPW + hl;
-            if (head < heads_kind) {
-                if (KVFP8 && !is_q) {
-                    uint8_t *dst = static_cast<uint8_t *>(a.k_cache) + (slot * a.hk + head) * D;
-                    if (kdiv.fast) {
-#pragma unroll
-                        for (int i = 0; i < CPL; ++i)
-                            *reinterpret_cast<u32x2 *>(dst + 8 * cid[i]) = quantize_chunk<T, true>(o[i], kdiv);
-                    } else {
-#pragma unroll 1
-                        for (int i = 0; i < CPL; ++i)
-                            *reinterpret_cast<u32x2 *>(dst + 8 * cid[i]) = quantize_chunk<T, false>(o[i], kdiv);
-                    }
-                } else {
-                    // one store sequence for every 16-bit destination; `out_row` is wave-uniform
-#pragma unroll
-                    for (int i = 0; i < CPL; ++i) *reinterpret_cast<u32x4 *>(out_row + (int64_t)head * D + 8 * cid[i]) = o[i];
-                }
-            }
-        }
-    } else {
-        // ------------------------------------------------------------------ V heads (set_kv only): copy or quantise
-        if constexpr (SETKV) {
-            const int round0 = (u - a.units_q - a.units_k) * a.rounds_per_wave;
-            const int rounds_kind = (a.hv + HPW - 1) / HPW;
-            const int round1 = min(round0 + (int)a.rounds_per_wave, rounds_kind);
-            const int64_t slot = a.kv_loc[t];
-            const Divider vdiv(a.v_scale);
-            for (int round = round0; round < round1; ++round) {
-                const int head = round * HPW + hl;
-                if (head >= a.hv) continue;
-                const uint16_t *src = token_in + (int64_t)(a.hq + a.hk + head) * D;
-                const int64_t off = (slot * a.hv + head) * D;
-                if constexpr (!KVFP8) {
-                    // chunk i*LPH + sub: every load / store instruction covers LPH*16 contiguous bytes per head
-                    u32x4 v[CPL];
-#pragma unroll
-                    for (int i = 0; i < CPL; ++i)
-                        v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 8 * (i * LPH + sub)));
-                    uint16_t *dst = static_cast<uint16_t *>(a.v_cache) + off;
-#pragma unroll
-                    for (int i = 0; i < CPL; ++i) *reinterpret_cast<u32x4 *>(dst + 8 * (i * LPH + sub)) = v[i];
-                } else {
-                    // adjacent chunk pairs {2sub, 2sub+1} (+ 2*LPH per further pair): 16 codes leave as one 16-byte store
-                    u32x4 v[CPL];
-#pragma unroll
-                    for (int i = 0; i < CPL; ++i)
-                        v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 8 * (2 * sub + (i & 1) + (i >> 1) * 2 * LPH)));
-                    uint8_t *dst = static_cast<uint8_t *>(a.v_cache) + off;
-                    if (vdiv.fast) {
-#pragma unroll
-                        for (int h = 0; h < CPL / 2; ++h) {
-                            const u32x2 qa = quantize_chunk<T, true>(v[2 * h], vdiv), qb = quantize_chunk<T, true>(v[2 * h + 1], vdiv);
-                            *reinterpret_cast<u32x4 *>(dst + 8 * (2 * sub + h * 2 * LPH)) = u32x4{qa[0], qa[1], qb[0], qb[1]};
-                        }
-                    } else {
-#pragma unroll 1
-                        for (int h = 0; h < CPL / 2; ++h) {
-                            const u32x2 qa = quantize_chunk<T, false>(v[2 * h], vdiv), qb = quantize_chunk<T, false>(v[2 * h + 1], vdiv);
-                            *reinterpret_cast<u32x4 *>(dst + 8 * (2 * sub + h * 2 * LPH)) = u32x4{qa[0], qa[1], qb[0], qb[1]};
-                        }
-                    }
+                    const uint32_t m1 = halves_mask(b1 >> (2 * j)), m2 = halves_mask(b2 >> (2 * j));
+                    st.cosv[j] = bitselect(m2, cos2[j], bitselect(m1, cos1[j], st.cosv[j]));
+                    st.sinv[j] = bitselect(m2, sin2[j], bitselect(m1, sin1[j], st.sinv[j]));
                 }
             }
         }
     }
+
+    // Norm, rotation and all stores of the unit.
+    static __device__ __forceinline__ void finish(const RopeArgs &a, int lane, UnitState &st) {
+        if (!st.live) return;
+        const int sub = lane % LPH;
+        const int heads_qk = a.hq + a.hk, heads_all = heads_qk + a.hv;
+        const u32x4 &xa = st.xa, &xb = st.xb, &wa = st.wa, &wb = st.wb, &cosv = st.cosv, &sinv = st.sinv;
+
+        // RMSNorm over the head: LPH lanes x 16 elements
+        float ss0 = 0.f, ss1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            ss0 = P::add_squares(xa[j], ss0);
+            ss1 = P::add_squares(xb[j], ss1);
+        }
+        const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
+        const float rstd = 1.0f / sqrtf(sumsq * (1.0f / D) + a.eps);  // D is a power of two: the product is exact
+
+        u32x4 na, nb;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t ta = P::pack(P::lo(xa[j]) * rstd, P::hi(xa[j]) * rstd);
+            const uint32_t tb = P::pack(P::lo(xb[j]) * rstd, P::hi(xb[j]) * rstd);
+            na[j] = P::pack(P::lo(wa[j]) * P::lo(ta), P::hi(wa[j]) * P::hi(ta));
+            nb[j] = P::pack(P::lo(wb[j]) * P::lo(tb), P::hi(wb[j]) * P::hi(tb));
+        }
+
+        u32x4 oa, ob;
+        if constexpr (NEOX) {
+            // chunk a holds x1 for frequencies 8*sub .. 8*sub+7, chunk b the matching x2
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float x1l = P::lo(na[j]), x1h = P::hi(na[j]), x2l = P::lo(nb[j]), x2h = P::hi(nb[j]);
+                const float cl = P::lo(cosv[j]), ch = P::hi(cosv[j]), sl = P::lo(sinv[j]), sh = P::hi(sinv[j]);
+                const uint32_t t1 = P::pack(x1l * cl, x1h * ch), t2 = P::pack(x2l * sl, x2h * sh);
+                const uint32_t t3 = P::pack(x2l * cl, x2h * ch), t4 = P::pack(x1l * sl, x1h * sh);
+                oa[j] = P::pack(P::lo(t1) - P::lo(t2), P::hi(t1) - P::hi(t2));
+                ob[j] = P::pack(P::lo(t3) + P::lo(t4), P::hi(t3) + P::hi(t4));
+            }
+        } else {
+            // each dword is one (x1, x2) pair; chunk a uses the lane's frequencies 0-3, chunk b 4-7
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                {
+                    const float x1 = P::lo(na[e]), x2 = P::hi(na[e]);
+                    const float c = elem<T>(cosv, e), s = elem<T>(sinv, e);
+                    const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
+                    oa[e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
+                }
+                {
+                    const float x1 = P::lo(nb[e]), x2 = P::hi(nb[e]);
+                    const float c = elem<T>(cosv, 4 + e), s = elem<T>(sinv, 4 + e);
+                    const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
+                    ob[e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
+                }
+            }
+        }
+
+        const int head = st.head;
+        if (st.active) {
+            if constexpr (!SETKV) {
+                uint16_t *dst = static_cast<uint16_t *>(a.qkv_out) + ((int64_t)st.t * heads_all + head) * D;
+                *reinterpret_cast<u32x4 *>(dst + c0(sub)) = oa;
+                *reinterpret_cast<u32x4 *>(dst + c1(sub)) = ob;
+            } else if (KVFP8 && !st.is_q) {
+                uint8_t *dst = static_cast<uint8_t *>(a.k_cache) + (st.slot * a.hk + (head - a.hq)) * D;
+                const float s = a.k_scale, rcp = 1.0f / s;
+                if (scale_is_fast(s)) {
+                    *reinterpret_cast<u32x2 *>(dst + c0(sub)) = quantize_chunk<T, true>(oa, s, rcp);
+                    *reinterpret_cast<u32x2 *>(dst + c1(sub)) = quantize_chunk<T, true>(ob, s, rcp);
+                } else {
+                    *reinterpret_cast<u32x2 *>(dst + c0(sub)) = quantize_chunk<T, false>(oa, s, rcp);
+                    *reinterpret_cast<u32x2 *>(dst + c1(sub)) = quantize_chunk<T, false>(ob, s, rcp);
+                }
+            } else {
+                // q_out row or (16-bit) K cache row of the slot: one store sequence, destination chosen per lane
+                uint16_t *dst = st.is_q ? static_cast<uint16_t *>(a.q_out) + ((int64_t)st.t * a.hq + head) * D
+                                        : static_cast<uint16_t *>(a.k_cache) + (st.slot * a.hk + (head - a.hq)) * D;
+                *reinterpret_cast<u32x4 *>(dst + c0(sub)) = oa;
+                *reinterpret_cast<u32x4 *>(dst + c1(sub)) = ob;
+            }
+        }
+
+        if constexpr (SETKV) {
+            // V: copied (16-bit cache) or quantised (fp8 cache), chunk by chunk
+            const int v_chunks = a.hv * (D / 8), v_first = st.u * 64 + lane;
+            const int stride = a.units_per_token * 64;
+            const float s = a.v_scale, rcp = 1.0f / s;
+            const bool fast = scale_is_fast(s);
+            u32x4 vchunk = st.vchunk;
+            for (int c = v_first; c < v_chunks; c += stride) {
+                if (c != v_first)
+                    vchunk = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(st.token_in + (int64_t)heads_qk * D + 8 * c));
+                const int64_t off = st.slot * a.hv * D + 8 * (int64_t)c;
+                if constexpr (!KVFP8) {
+                    *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(a.v_cache) + off) = vchunk;
+                } else {
+                    *reinterpret_cast<u32x2 *>(static_cast<uint8_t *>(a.v_cache) + off) =
+                        fast ? quantize_chunk<T, true>(vchunk, s, rcp) : quantize_chunk<T, false>(vchunk, s, rcp);
+                }
+            }
+        }
+    }
+};
+
+// UPW: units per wave.  With 2, a wave has the loads of two units in flight before it starts on the first.
+template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8, int UPW>
+__global__ void __launch_bounds__(512) rope_rms_kernel(const RopeArgs a) {
+    using Unit = RopeUnit<T, D, NEOX, AXES, SETKV, KVFP8>;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t unit0 = (blockIdx.x * (blockDim.x >> 6) + wave) * UPW;
+    if (unit0 >= a.total_units) return;
+    const int lane = threadIdx.x & 63;
+    UnitState st[UPW];
+#pragma unroll
+    for (int i = 0; i < UPW; ++i) Unit::issue_loads(a, unit0 + i, lane, st[i]);
+    // Every load of the wave is in flight before the first use of any of them: without this fence the scheduler
+    // moves arithmetic above later loads and the wave pays several memory round trips in a row.
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < UPW; ++i) Unit::finish(a, lane, st[i]);
 }
 
 int g_block_threads = 0;    // 0 = default
-int g_rounds_per_wave = 0;  // 0 = heuristic
-int g_chunks_per_lane = 2;  // 2 or 4
+int g_units_per_wave = 0;   // 0 = heuristic, else 1 or 2
 
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 int launch_one(const RopeArgs &a, hipStream_t stream) {
     const int threads = g_block_threads ? g_block_threads : 256;
-    const uint32_t waves_per_block = threads / 64;
-    const uint32_t blocks = (a.total_units + waves_per_block - 1) / waves_per_block;
-    if (g_chunks_per_lane == 4)
-        rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8, 4><<<blocks, threads, 0, stream>>>(a);
-    else
+    const int upw = g_units_per_wave ? g_units_per_wave : 1;
+    const uint32_t units_per_block = threads / 64 * upw;
+    const uint32_t blocks = (a.total_units + units_per_block - 1) / units_per_block;
+    if (upw == 2)
         rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8, 2><<<blocks, threads, 0, stream>>>(a);
+    else
+        rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8, 1><<<blocks, threads, 0, stream>>>(a);
     return hip_status(hipGetLastError());
 }
 
@@ -440,19 +369,19 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     if (!aligned16(qkv_in) || !aligned16(qw) || !aligned16(kw) || !aligned16(cos_sin)) return GPUK_ERR_MISALIGNED;
     const bool kv_fp8 = set_kv && kv_dtype == GPUK_KV_E4M3FN;
     if (set_kv) {
-        if (!q_out || !k_cache || !v_cache || !kv_loc) return GPUK_ERR_INVALID_ARG;
+        // a buffer may be absent (or empty) when no head of its kind exists
+        if ((hq > 0 && !q_out) || (hk > 0 && !k_cache) || (hv > 0 && !v_cache) || !kv_loc) return GPUK_ERR_INVALID_ARG;
         if (!aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache)) return GPUK_ERR_MISALIGNED;
         if (kv_fp8 && !(k_scale > 0.f && v_scale > 0.f)) return GPUK_ERR_INVALID_ARG;
     }
-    // Heads per wave-round, rounds per kind, and how many rounds one wave takes on.  One round per wave
-    // measured fastest at every size tried (more waves in flight hide the position -> cos/sin dependent loads
-    // better than a longer wave with a one-round prefetch does); larger values stay selectable for tuning.
-    const int64_t hpw = 64 / (D / (8 * g_chunks_per_lane));
-    const int64_t rq = (hq + hpw - 1) / hpw, rk = (hk + hpw - 1) / hpw, rv = set_kv ? (hv + hpw - 1) / hpw : 0;
-    const int64_t rpw = g_rounds_per_wave ? g_rounds_per_wave : 1;
-    const int64_t uq = (rq + rpw - 1) / rpw, uk = (rk + rpw - 1) / rpw, uv = (rv + rpw - 1) / rpw;
-    const int64_t upt = uq + uk + uv;
-    if (upt * T >= 0x7fffffffLL) return GPUK_ERR_UNSUPPORTED;
+    // one wave per group of 64/(D/16) consecutive Q/K heads of a token; with a KV cache and no Q/K heads at all the
+    // token still gets the waves its V row needs
+    const int64_t hpw = 64 / (D / 16);
+    int64_t upt = (hq + hk + hpw - 1) / hpw;
+    if (upt == 0) upt = (hv * (D / 8) + 63) / 64;
+    if (hq + hk == 0) return GPUK_ERR_UNSUPPORTED;  // a qkv row without Q and K heads has nothing to rotate
+    // mulhi(unit, ceil(2^32/upt)) equals unit / upt while unit * upt < 2^32
+    if (upt * T >= 0x7fffffffLL || upt * T * upt >= (1LL << 32)) return GPUK_ERR_UNSUPPORTED;
     a.qkv_in = qkv_in;
     a.qkv_out = qkv_out;
     a.qw = qw;
@@ -467,9 +396,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     a.kv_loc = kv_loc;
     a.total_units = (uint32_t)(upt * T);
     a.units_per_token = (uint32_t)upt;
-    a.units_q = (uint32_t)uq;
-    a.units_k = (uint32_t)uk;
-    a.rounds_per_wave = (uint32_t)rpw;
+    a.upt_magic = upt == 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)upt - 1) / (uint64_t)upt);
     a.hq = (int)hq;
     a.hk = (int)hk;
     a.hv = (int)hv;
@@ -485,8 +412,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
 
 void set_rope_tuning(int key, int value) {
     if (key == 0) g_block_threads = value;
-    if (key == 1) g_rounds_per_wave = value;
-    if (key == 2) g_chunks_per_lane = value;
+    if (key == 1) g_units_per_wave = value;
 }
 
 }  // namespace gpuk

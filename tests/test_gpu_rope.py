@@ -146,20 +146,18 @@ def test_rope_set_kv_head_mixes(device, hq, hk, hv, fp8):
     check_set_kv(inp, run_set_kv(inp, device), f"[set_kv {hq},{hk},{hv}]")
 
 
-@pytest.mark.parametrize("chunks_per_lane,rounds_per_wave,threads", [(2, 1, 128), (2, 4, 256), (4, 1, 256), (4, 3, 512), (2, 64, 64)])
-def test_launch_shape_variants(device, chunks_per_lane, rounds_per_wave, threads):
-    """Every selectable work decomposition (chunks per lane, rounds per wave, workgroup size) gives the same
-    bits as the oracle; the defaults are only the fastest of them."""
+@pytest.mark.parametrize("threads,units_per_wave", [(64, 1), (128, 2), (512, 1), (256, 2)])
+def test_launch_shape_variants(device, threads, units_per_wave):
+    """Workgroup size and units per wave are tuning choices only: every setting gives the same bits as the oracle."""
     from gpuk_amd import capi
 
-    print(f"case variants cpl={chunks_per_lane} rpw={rounds_per_wave} threads={threads}", flush=True)
-    capi.set_tuning("rope_chunks_per_lane", chunks_per_lane)
-    capi.set_tuning("rope_rounds_per_wave", rounds_per_wave)
+    print(f"case variants threads={threads} units_per_wave={units_per_wave}", flush=True)
     capi.set_tuning("rope_block_threads", threads)
+    capi.set_tuning("rope_units_per_wave", units_per_wave)
     try:
         for hs, neox, mrope, fp8, heads in ((128, True, False, False, (32, 8, 8)), (64, False, True, True, (20, 20, 20)),
                                             (256, True, True, False, (9, 3, 3)), (128, False, False, True, (64, 8, 8))):
-            inp = make(45, heads[0], hs, neox, seed=hs + rounds_per_wave, mrope=mrope, interleaved=mrope, fp8=fp8,
+            inp = make(45, heads[0], hs, neox, seed=hs + threads, mrope=mrope, interleaved=mrope, fp8=fp8,
                        hk=heads[1], hv=heads[2])
             check_set_kv(inp, run_set_kv(inp, device), f"[variant D={hs}]")
             got = run_inplace(inp, device)
@@ -168,9 +166,17 @@ def test_launch_shape_variants(device, chunks_per_lane, rounds_per_wave, threads
             assert_rotated_close(got[:, :nqk], want[:, :nqk], "in place q,k")
             assert_bits_equal(got[:, nqk:], want[:, nqk:], "in place v")
     finally:
-        capi.set_tuning("rope_chunks_per_lane", 2)
-        capi.set_tuning("rope_rounds_per_wave", 0)
         capi.set_tuning("rope_block_threads", 0)
+        capi.set_tuning("rope_units_per_wave", 0)
+
+
+@pytest.mark.parametrize("hq,hk,hv,head_size", [(3, 1, 40, 64), (1, 1, 17, 256), (7, 2, 0, 128), (2, 9, 33, 128)])
+def test_value_heads_outnumber_the_waves(device, hq, hk, hv, head_size):
+    """The V row is shared out over the waves that rotate Q and K; with few Q/K heads and many V heads each wave
+    walks several strides of it, with none the V part is empty."""
+    for fp8 in (False, True):
+        inp = make(29, hq, head_size, True, seed=hv + head_size, fp8=fp8, hk=hk, hv=hv)
+        check_set_kv(inp, run_set_kv(inp, device), f"[V-heavy {hq},{hk},{hv} D={head_size} fp8={fp8}]")
 
 
 def test_config3_qwen3_like(device):
