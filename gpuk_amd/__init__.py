@@ -35,6 +35,7 @@ allreduce_rms = torch.ops.gpuk.allreduce_rms
 fused_rope_rms = torch.ops.gpuk.fused_rope_rms
 fused_mrope_3d_rms = torch.ops.gpuk.fused_mrope_3d_rms
 fused_mrope_3d_rms_set_kv = torch.ops.gpuk.fused_mrope_3d_rms_set_kv
+fused_rope_rms_2way = torch.ops.gpuk.fused_rope_rms_2way
 fused_rope_rms_set_kv = torch.ops.gpuk.fused_rope_rms_set_kv       # additive: 1-D positions + KV write
 set_fp8_max = torch.ops.gpuk.set_fp8_max                           # additive
 get_fp8_max = torch.ops.gpuk.get_fp8_max                           # additive

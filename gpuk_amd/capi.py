@@ -14,7 +14,7 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libgpuk_amd.so")
 
 EXPORTS = ("gpuk_status_string", "gpuk_abi_version", "gpuk_add_rmsnorm_quant", "gpuk_rope_rms",
-           "gpuk_rope_rms_set_kv", "gpuk_copy_bytes", "gpuk_set_tuning")
+           "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_set_tuning")
 
 DTYPE = {torch.bfloat16: 0, torch.float16: 1}
 QUANT_NONE, QUANT_FP8_DYNAMIC, QUANT_FP8_E4M3FNUZ, QUANT_FP8_STATIC = 0, 1, 2, 3
@@ -50,6 +50,9 @@ def lib():
         L.gpuk_rope_rms.argtypes = rope_head + [C.c_void_p]
         L.gpuk_rope_rms_set_kv.restype = C.c_int
         L.gpuk_rope_rms_set_kv.argtypes = rope_head + [C.c_void_p] * 4 + [C.c_float, C.c_float, C.c_int, C.c_void_p]
+        L.gpuk_rope_rms_2way.restype = C.c_int
+        L.gpuk_rope_rms_2way.argtypes = [C.c_void_p] * 10 + [C.c_int64] * 6 + [C.c_int, C.c_float, C.c_int,
+                                                                             C.c_void_p, C.c_void_p, C.c_void_p]
         L.gpuk_copy_bytes.restype = C.c_int
         L.gpuk_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
         _lib = L
@@ -120,3 +123,13 @@ def copy_bytes(dst, src, nbytes: int, stream=None) -> None:
     rc = lib().gpuk_copy_bytes(_ptr(dst), _ptr(src), nbytes, _stream(stream))
     if rc:
         raise GpukError(rc, "gpuk_copy_bytes")
+
+
+def rope_rms_2way(q0, k0, q1, k1, w_q0, w_k0, w_q1, w_k1, cos_sin0, cos_sin1, batch_size, T0, T1, Hq, Hk, D,
+                  is_interleaved, eps, out_q01, out_k01, stream=None) -> None:
+    rc = lib().gpuk_rope_rms_2way(_ptr(q0), _ptr(k0), _ptr(q1), _ptr(k1), _ptr(w_q0), _ptr(w_k0), _ptr(w_q1),
+                                  _ptr(w_k1), _ptr(cos_sin0), _ptr(cos_sin1), batch_size, T0, T1, Hq, Hk, D,
+                                  int(is_interleaved), eps, DTYPE[q0.dtype], _ptr(out_q01), _ptr(out_k01),
+                                  _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_rope_rms_2way")

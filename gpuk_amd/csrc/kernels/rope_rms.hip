@@ -21,6 +21,8 @@
 //     fp8 cache: code = e4m3fn(rT(o / scale)), saturating at +-448
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "../../../include/gpuk_amd.h"
 #include "device_utils.h"
 #include "host_utils.h"
@@ -81,6 +83,61 @@ __device__ __forceinline__ u32x2 quantize_chunk(const u32x4 &v, float scale, flo
     return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
 }
 __device__ __forceinline__ bool scale_is_fast(float s) { return s >= 0x1p-60f && s <= 0x1p60f; }
+
+// RMSNorm of one head (D/16 lanes x two chunks) followed by the rotation, for the lane's two chunks.
+//   NeoX : chunk a holds x1 for the lane's 8 frequencies, chunk b the matching x2.
+//   GPT-J: each dword is one (x1, x2) pair; chunk a uses the lane's frequencies 0-3, chunk b 4-7.
+template <typename T, int D, bool NEOX>
+__device__ __forceinline__ void norm_rotate(const u32x4 &xa, const u32x4 &xb, const u32x4 &wa, const u32x4 &wb,
+                                            const u32x4 &cosv, const u32x4 &sinv, float eps, u32x4 &oa, u32x4 &ob) {
+    using P = Pack16<T>;
+    constexpr int LPH = D / 16;
+    float ss0 = 0.f, ss1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        ss0 = P::add_squares(xa[j], ss0);
+        ss1 = P::add_squares(xb[j], ss1);
+    }
+    const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
+    const float rstd = 1.0f / sqrtf(sumsq * (1.0f / D) + eps);  // D is a power of two: the product is exact
+
+    u32x4 na, nb;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t ta = P::pack(P::lo(xa[j]) * rstd, P::hi(xa[j]) * rstd);
+        const uint32_t tb = P::pack(P::lo(xb[j]) * rstd, P::hi(xb[j]) * rstd);
+        na[j] = P::pack(P::lo(wa[j]) * P::lo(ta), P::hi(wa[j]) * P::hi(ta));
+        nb[j] = P::pack(P::lo(wb[j]) * P::lo(tb), P::hi(wb[j]) * P::hi(tb));
+    }
+
+    if constexpr (NEOX) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float x1l = P::lo(na[j]), x1h = P::hi(na[j]), x2l = P::lo(nb[j]), x2h = P::hi(nb[j]);
+            const float cl = P::lo(cosv[j]), ch = P::hi(cosv[j]), sl = P::lo(sinv[j]), sh = P::hi(sinv[j]);
+            const uint32_t t1 = P::pack(x1l * cl, x1h * ch), t2 = P::pack(x2l * sl, x2h * sh);
+            const uint32_t t3 = P::pack(x2l * cl, x2h * ch), t4 = P::pack(x1l * sl, x1h * sh);
+            oa[j] = P::pack(P::lo(t1) - P::lo(t2), P::hi(t1) - P::hi(t2));
+            ob[j] = P::pack(P::lo(t3) + P::lo(t4), P::hi(t3) + P::hi(t4));
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            {
+                const float x1 = P::lo(na[e]), x2 = P::hi(na[e]);
+                const float c = elem<T>(cosv, e), s = elem<T>(sinv, e);
+                const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
+                oa[e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
+            }
+            {
+                const float x1 = P::lo(nb[e]), x2 = P::hi(nb[e]);
+                const float c = elem<T>(cosv, 4 + e), s = elem<T>(sinv, 4 + e);
+                const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
+                ob[e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
+            }
+        }
+    }
+}
 
 // What one wave keeps about one unit (= one group of 64/(D/16) consecutive Q/K heads of one token, plus its share
 // of the token's V row) between issuing the unit's loads and finishing it.
@@ -170,55 +227,8 @@ struct RopeUnit {
         const int heads_qk = a.hq + a.hk, heads_all = heads_qk + a.hv;
         const u32x4 &xa = st.xa, &xb = st.xb, &wa = st.wa, &wb = st.wb, &cosv = st.cosv, &sinv = st.sinv;
 
-        // RMSNorm over the head: LPH lanes x 16 elements
-        float ss0 = 0.f, ss1 = 0.f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            ss0 = P::add_squares(xa[j], ss0);
-            ss1 = P::add_squares(xb[j], ss1);
-        }
-        const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
-        const float rstd = 1.0f / sqrtf(sumsq * (1.0f / D) + a.eps);  // D is a power of two: the product is exact
-
-        u32x4 na, nb;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t ta = P::pack(P::lo(xa[j]) * rstd, P::hi(xa[j]) * rstd);
-            const uint32_t tb = P::pack(P::lo(xb[j]) * rstd, P::hi(xb[j]) * rstd);
-            na[j] = P::pack(P::lo(wa[j]) * P::lo(ta), P::hi(wa[j]) * P::hi(ta));
-            nb[j] = P::pack(P::lo(wb[j]) * P::lo(tb), P::hi(wb[j]) * P::hi(tb));
-        }
-
         u32x4 oa, ob;
-        if constexpr (NEOX) {
-            // chunk a holds x1 for frequencies 8*sub .. 8*sub+7, chunk b the matching x2
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float x1l = P::lo(na[j]), x1h = P::hi(na[j]), x2l = P::lo(nb[j]), x2h = P::hi(nb[j]);
-                const float cl = P::lo(cosv[j]), ch = P::hi(cosv[j]), sl = P::lo(sinv[j]), sh = P::hi(sinv[j]);
-                const uint32_t t1 = P::pack(x1l * cl, x1h * ch), t2 = P::pack(x2l * sl, x2h * sh);
-                const uint32_t t3 = P::pack(x2l * cl, x2h * ch), t4 = P::pack(x1l * sl, x1h * sh);
-                oa[j] = P::pack(P::lo(t1) - P::lo(t2), P::hi(t1) - P::hi(t2));
-                ob[j] = P::pack(P::lo(t3) + P::lo(t4), P::hi(t3) + P::hi(t4));
-            }
-        } else {
-            // each dword is one (x1, x2) pair; chunk a uses the lane's frequencies 0-3, chunk b 4-7
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                {
-                    const float x1 = P::lo(na[e]), x2 = P::hi(na[e]);
-                    const float c = elem<T>(cosv, e), s = elem<T>(sinv, e);
-                    const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
-                    oa[e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
-                }
-                {
-                    const float x1 = P::lo(nb[e]), x2 = P::hi(nb[e]);
-                    const float c = elem<T>(cosv, 4 + e), s = elem<T>(sinv, 4 + e);
-                    const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
-                    ob[e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
-                }
-            }
-        }
+        norm_rotate<T, D, NEOX>(xa, xb, wa, wb, cosv, sinv, a.eps, oa, ob);
 
         const int head = st.head;
         if (st.active) {
@@ -283,6 +293,87 @@ __global__ void __launch_bounds__(512) rope_rms_kernel(const RopeArgs a) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < UPW; ++i) Unit::finish(a, lane, st[i]);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Two token streams with their own norm weights and per-token cos/sin rows, outputs concatenated along the token
+// axis (reference: fused_rope_rms_2way, src/ops/fused_rope.cpp:168-227 -> src/impl/rope_rms_impl.h:612-857).
+// Per batch entry there are four segments of heads, each a contiguous [tokens, heads, D] block:
+//   0: q0 -> out_q[:, 0:T0]   1: k0 -> out_k[:, 0:T0]   2: q1 -> out_q[:, T0:T0+T1]   3: k1 -> out_k[:, T0:T0+T1]
+// A wave takes 64/(D/16) consecutive heads of one segment (they may belong to several tokens, so the cos/sin row
+// is chosen per lane); blockIdx.y is the batch entry.
+struct TwoWayArgs {
+    const void *in[4];     // q0, k0, q1, k1
+    const void *w[4];      // w_q0, w_k0, w_q1, w_k1
+    const void *cos_sin[2];
+    void *out[2];          // out_q01, out_k01
+    uint32_t unit_end[4];  // prefix sums of the segments' unit counts
+    uint32_t rows[4];      // tokens * heads of each segment
+    uint32_t heads[2];     // Hq, Hk
+    uint32_t heads_magic[2];  // ceil(2^32 / heads), 0 for heads == 1
+    int tokens0, tokens1;
+    float eps;
+};
+
+template <typename T, int D, bool NEOX>
+__global__ void __launch_bounds__(256) rope_rms_2way_kernel(const TwoWayArgs a) {
+    constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t unit = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (unit >= a.unit_end[3]) return;
+    const int seg = (unit >= a.unit_end[0]) + (unit >= a.unit_end[1]) + (unit >= a.unit_end[2]);  // wave-uniform
+    const uint32_t unit_in_seg = unit - (seg ? a.unit_end[seg - 1] : 0u);
+    const int kind = seg & 1, stream_id = seg >> 1;  // q|k, stream 0|1
+    const uint32_t heads = a.heads[kind], rows = a.rows[seg];
+    const int tokens_seg = stream_id ? a.tokens1 : a.tokens0;
+    const int batch = blockIdx.y;
+
+    const int lane = threadIdx.x & 63, sub = lane % LPH, hl = lane / LPH;
+    const uint32_t row_raw = unit_in_seg * HPW + hl;
+    const bool active = row_raw < rows;
+    const uint32_t row = min(row_raw, rows - 1);  // (token, head) flattened inside the segment
+    const uint32_t token = a.heads_magic[kind] ? __umulhi(row, a.heads_magic[kind]) : row;
+    const uint32_t head = row - token * heads;
+
+    const int c0 = NEOX ? 8 * sub : 16 * sub, c1 = NEOX ? HALF + 8 * sub : 16 * sub + 8, fc = 8 * sub;
+    const uint16_t *src = static_cast<const uint16_t *>(a.in[seg]) + ((int64_t)batch * rows + row) * D;
+    const u32x4 xa = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c0));
+    const u32x4 xb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c1));
+    const uint16_t *wsrc = static_cast<const uint16_t *>(a.w[seg]);
+    const u32x4 wa = *reinterpret_cast<const u32x4 *>(wsrc + c0);
+    const u32x4 wb = *reinterpret_cast<const u32x4 *>(wsrc + c1);
+    const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin[stream_id]) + (int64_t)token * D;
+    const u32x4 cosv = *reinterpret_cast<const u32x4 *>(table + fc);
+    const u32x4 sinv = *reinterpret_cast<const u32x4 *>(table + HALF + fc);
+    __builtin_amdgcn_sched_barrier(0);
+
+    u32x4 oa, ob;
+    norm_rotate<T, D, NEOX>(xa, xb, wa, wb, cosv, sinv, a.eps, oa, ob);
+    if (active) {
+        const int64_t out_token = (int64_t)batch * (a.tokens0 + a.tokens1) + (stream_id ? a.tokens0 : 0) + token;
+        uint16_t *dst = static_cast<uint16_t *>(a.out[kind]) + (out_token * heads + head) * D;
+        *reinterpret_cast<u32x4 *>(dst + c0) = oa;
+        *reinterpret_cast<u32x4 *>(dst + c1) = ob;
+    }
+    (void)tokens_seg;
+}
+
+template <typename T, int D>
+int launch_2way(const TwoWayArgs &a, bool neox, unsigned batch, hipStream_t stream) {
+    const dim3 grid((a.unit_end[3] + 3) / 4, batch);
+    if (neox) rope_rms_2way_kernel<T, D, true><<<grid, 256, 0, stream>>>(a);
+    else rope_rms_2way_kernel<T, D, false><<<grid, 256, 0, stream>>>(a);
+    return hip_status(hipGetLastError());
+}
+
+template <typename T>
+int launch_2way_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned batch, hipStream_t stream) {
+    switch (D) {
+        case 64: return launch_2way<T, 64>(a, neox, batch, stream);
+        case 128: return launch_2way<T, 128>(a, neox, batch, stream);
+        case 256: return launch_2way<T, 256>(a, neox, batch, stream);
+        default: return GPUK_ERR_UNSUPPORTED;
+    }
 }
 
 int g_block_threads = 0;    // 0 = default
@@ -439,4 +530,56 @@ extern "C" int gpuk_rope_rms_set_kv(const void *qkv, const void *qw, const void 
                              num_tokens, num_heads_q, num_heads_k, num_heads_v, head_size, is_neox_style,
                              mrope_section, is_interleaved, eps, dtype, true, q_out, k_cache, v_cache, kv_loc,
                              k_scale, v_scale, kv_dtype, stream);
+}
+
+extern "C" int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1, const void *k1, const void *w_q0,
+                                  const void *w_k0, const void *w_q1, const void *w_k1, const void *cos_sin0,
+                                  const void *cos_sin1, int64_t batch_size, int64_t num_tokens0, int64_t num_tokens1,
+                                  int64_t num_heads_q, int64_t num_heads_k, int64_t head_size, int is_interleaved,
+                                  float eps, int dtype, void *out_q01, void *out_k01, void *stream) {
+    using namespace gpuk;
+    if (batch_size < 0 || num_tokens0 < 0 || num_tokens1 < 0 || num_heads_q < 0 || num_heads_k < 0) return GPUK_ERR_INVALID_ARG;
+    if (head_size != 64 && head_size != 128 && head_size != 256) return GPUK_ERR_UNSUPPORTED;
+    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16) return GPUK_ERR_UNSUPPORTED;
+    if (batch_size > 65535) return GPUK_ERR_UNSUPPORTED;  // grid.y
+    const int64_t hpw = 64 / (head_size / 16);
+    const int64_t rows[4] = {num_tokens0 * num_heads_q, num_tokens0 * num_heads_k, num_tokens1 * num_heads_q,
+                             num_tokens1 * num_heads_k};
+    const void *ins[4] = {q0, k0, q1, k1};
+    const void *ws[4] = {w_q0, w_k0, w_q1, w_k1};
+    TwoWayArgs a{};
+    int64_t end = 0;
+    for (int s = 0; s < 4; ++s) {
+        if (rows[s] >= (1LL << 31)) return GPUK_ERR_UNSUPPORTED;
+        if (rows[s] > 0 && (!ins[s] || !ws[s] || !aligned16(ins[s]) || !aligned16(ws[s])))
+            return !ins[s] || !ws[s] ? GPUK_ERR_INVALID_ARG : GPUK_ERR_MISALIGNED;
+        end += (rows[s] + hpw - 1) / hpw;
+        a.in[s] = ins[s];
+        a.w[s] = ws[s];
+        a.unit_end[s] = (uint32_t)end;
+        a.rows[s] = (uint32_t)rows[s];
+    }
+    if (end >= (1LL << 31)) return GPUK_ERR_UNSUPPORTED;
+    if (batch_size == 0 || end == 0) return GPUK_OK;
+    if ((num_tokens0 > 0 && !cos_sin0) || (num_tokens1 > 0 && !cos_sin1)) return GPUK_ERR_INVALID_ARG;
+    if ((rows[0] + rows[2] > 0 && !out_q01) || (rows[1] + rows[3] > 0 && !out_k01)) return GPUK_ERR_INVALID_ARG;
+    if (!aligned16(cos_sin0) || !aligned16(cos_sin1) || !aligned16(out_q01) || !aligned16(out_k01)) return GPUK_ERR_MISALIGNED;
+    a.cos_sin[0] = cos_sin0;
+    a.cos_sin[1] = cos_sin1;
+    a.out[0] = out_q01;
+    a.out[1] = out_k01;
+    const int64_t heads[2] = {num_heads_q, num_heads_k};
+    for (int k = 0; k < 2; ++k) {
+        a.heads[k] = (uint32_t)heads[k];
+        // mulhi(row, ceil(2^32/heads)) == row / heads while row * heads < 2^32
+        if (heads[k] > 1 && std::max(rows[k], rows[k + 2]) * heads[k] >= (1LL << 32)) return GPUK_ERR_UNSUPPORTED;
+        a.heads_magic[k] = heads[k] <= 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)heads[k] - 1) / (uint64_t)heads[k]);
+    }
+    a.tokens0 = (int)num_tokens0;
+    a.tokens1 = (int)num_tokens1;
+    a.eps = eps;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool neox = !is_interleaved;  // reference: fused_rope.cpp:168-227 dispatches the NeoX kernel when !is_interleaved
+    if (dtype == GPUK_DTYPE_BF16) return launch_2way_head_size<BF16>(a, head_size, neox, (unsigned)batch_size, s);
+    return launch_2way_head_size<FP16>(a, head_size, neox, (unsigned)batch_size, s);
 }

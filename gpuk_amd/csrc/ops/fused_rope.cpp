@@ -112,4 +112,53 @@ void fused_rope_rms_set_kv(Tensor &qkv, Tensor &qw, Tensor &kw, Tensor &cos_sin,
                num_heads_k, num_heads_v, head_size, is_neox_style, eps, q, k_cache, v_cache, kv_loc, k_scale, v_scale);
 }
 
+// fused_rope_rms_2way: shape inference shared by the Meta and the GPU kernel (src/ops/fused_rope.cpp:168-182).
+std::tuple<Tensor, Tensor> fused_rope_rms_2way_meta(Tensor &q0, Tensor &k0, Tensor &q1, Tensor &k1, Tensor &w_q0,
+                                                    Tensor &w_k0, Tensor &w_q1, Tensor &w_k1, Tensor &cos_sin0,
+                                                    Tensor &cos_sin1, int64_t batch_size, int64_t num_tokens0,
+                                                    int64_t num_tokens1, int64_t num_heads_q, int64_t num_heads_k,
+                                                    int64_t head_size, bool is_interleaved, double eps) {
+    TORCH_CHECK(q0.is_contiguous() && k0.is_contiguous() && q1.is_contiguous() && k1.is_contiguous());
+    TORCH_CHECK(w_q0.is_contiguous() && w_k0.is_contiguous() && w_q1.is_contiguous() && w_k1.is_contiguous());
+    TORCH_CHECK(cos_sin0.is_contiguous() && cos_sin1.is_contiguous());
+    Tensor out_q01 = at::empty({batch_size, num_tokens0 + num_tokens1, num_heads_q, head_size}, q0.options());
+    Tensor out_k01 = at::empty({batch_size, num_tokens0 + num_tokens1, num_heads_k, head_size}, k0.options());
+    return std::make_tuple(std::move(out_q01), std::move(out_k01));
+}
+
+std::tuple<Tensor, Tensor> fused_rope_rms_2way(Tensor &q0, Tensor &k0, Tensor &q1, Tensor &k1, Tensor &w_q0, Tensor &w_k0,
+                                               Tensor &w_q1, Tensor &w_k1, Tensor &cos_sin0, Tensor &cos_sin1,
+                                               int64_t batch_size, int64_t num_tokens0, int64_t num_tokens1,
+                                               int64_t num_heads_q, int64_t num_heads_k, int64_t head_size,
+                                               bool is_interleaved, double eps) {
+    const char *op = "fused_rope_rms_2way";
+    auto outs = fused_rope_rms_2way_meta(q0, k0, q1, k1, w_q0, w_k0, w_q1, w_k1, cos_sin0, cos_sin1, batch_size,
+                                         num_tokens0, num_tokens1, num_heads_q, num_heads_k, head_size, is_interleaved, eps);
+    TORCH_CHECK(head_size == 64 || head_size == 128 || head_size == 256, op, ": head_size must be 64, 128 or 256");
+    TORCH_CHECK(q0.numel() == batch_size * num_tokens0 * num_heads_q * head_size &&
+                    k0.numel() == batch_size * num_tokens0 * num_heads_k * head_size &&
+                    q1.numel() == batch_size * num_tokens1 * num_heads_q * head_size &&
+                    k1.numel() == batch_size * num_tokens1 * num_heads_k * head_size,
+                op, ": q0/k0/q1/k1 must be [batch, tokens, heads, head_size]");
+    TORCH_CHECK(w_q0.numel() == head_size && w_k0.numel() == head_size && w_q1.numel() == head_size &&
+                    w_k1.numel() == head_size, op, ": the norm weights must hold head_size elements");
+    TORCH_CHECK(cos_sin0.numel() == num_tokens0 * head_size && cos_sin1.numel() == num_tokens1 * head_size, op,
+                ": cos_sin0/1 must be [num_tokens, head_size]");
+    const auto act = q0.scalar_type();
+    for (const Tensor *t : {&k0, &q1, &k1, &w_q0, &w_k0, &w_q1, &w_k1, &cos_sin0, &cos_sin1}) {
+        TORCH_CHECK(t->scalar_type() == act, op, ": all tensors must share q0's dtype");
+        TORCH_CHECK(t->device() == q0.device(), op, ": all tensors must be on the same device");
+    }
+    TORCH_CHECK(q0.is_cuda(), op, ": tensors must live on the GPU");
+    const int dtype = activation_dtype(q0, op);
+    DeviceGuard guard(q0.device());
+    const int status = gpuk_rope_rms_2way(q0.data_ptr(), k0.data_ptr(), q1.data_ptr(), k1.data_ptr(), w_q0.data_ptr(),
+                                          w_k0.data_ptr(), w_q1.data_ptr(), w_k1.data_ptr(), cos_sin0.data_ptr(),
+                                          cos_sin1.data_ptr(), batch_size, num_tokens0, num_tokens1, num_heads_q,
+                                          num_heads_k, head_size, is_interleaved, (float)eps, dtype,
+                                          std::get<0>(outs).data_ptr(), std::get<1>(outs).data_ptr(), current_stream());
+    check_status(status, op);
+    return outs;
+}
+
 }  // namespace gpuk_ops

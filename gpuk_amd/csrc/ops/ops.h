@@ -10,6 +10,7 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/library.h>
 
+#include <tuple>
 #include <vector>
 
 #include "../../../include/gpuk_amd.h"
@@ -56,5 +57,18 @@ void fused_rope_rms_set_kv(Tensor &qkv, Tensor &qw, Tensor &kw, Tensor &cos_sin,
                            int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
                            int64_t head_size, bool is_neox_style, double eps, Tensor &q, Tensor &k_cache,
                            Tensor &v_cache, Tensor &kv_loc, double k_scale, double v_scale);
+
+// Two token streams, outputs concatenated along the token axis (functional op with a Meta kernel, as in the
+// reference: src/ops/ops.h:52-65).
+std::tuple<Tensor, Tensor> fused_rope_rms_2way_meta(Tensor &q0, Tensor &k0, Tensor &q1, Tensor &k1, Tensor &w_q0,
+                                                    Tensor &w_k0, Tensor &w_q1, Tensor &w_k1, Tensor &cos_sin0,
+                                                    Tensor &cos_sin1, int64_t batch_size, int64_t num_tokens0,
+                                                    int64_t num_tokens1, int64_t num_heads_q, int64_t num_heads_k,
+                                                    int64_t head_size, bool is_interleaved, double eps);
+std::tuple<Tensor, Tensor> fused_rope_rms_2way(Tensor &q0, Tensor &k0, Tensor &q1, Tensor &k1, Tensor &w_q0, Tensor &w_k0,
+                                               Tensor &w_q1, Tensor &w_k1, Tensor &cos_sin0, Tensor &cos_sin1,
+                                               int64_t batch_size, int64_t num_tokens0, int64_t num_tokens1,
+                                               int64_t num_heads_q, int64_t num_heads_k, int64_t head_size,
+                                               bool is_interleaved, double eps);
 
 }  // namespace gpuk_ops

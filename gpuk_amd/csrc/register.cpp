@@ -1,7 +1,7 @@
 // Operator registration of the `gpuk` torch library for the two fused paths.
 //
-// The four schema strings marked "reference" are the reference's own (src/register.cpp:37-39, :42-44,
-// :47-49, :52-55), so `torch.ops.gpuk.<name>(...)` call sites keep working unchanged.  Compute ops are
+// The five schema strings marked "reference" are the reference's own (src/register.cpp:37-39, :42-44,
+// :47-49, :52-55, :58-61), so `torch.ops.gpuk.<name>(...)` call sites keep working unchanged.  Compute ops are
 // registered for the CUDA dispatch key, which is the key HIP tensors carry on PyTorch-ROCm.
 #include "ops/ops.h"
 
@@ -38,6 +38,14 @@ TORCH_LIBRARY(gpuk, m) {
           "bool is_neox_style, float eps, Tensor q, Tensor k_cache, Tensor v_cache, Tensor kv_loc, float k_scale, "
           "float v_scale) -> ()");
     m.impl("fused_rope_rms_set_kv", c10::DispatchKey::CUDA, &fused_rope_rms_set_kv);
+
+    // reference: src/register.cpp:58-63 (functional op with a Meta kernel for shape inference)
+    m.def("fused_rope_rms_2way(Tensor q0, Tensor k0, Tensor q1, Tensor k1, Tensor w_q0, Tensor w_k0, Tensor w_q1, "
+          "Tensor w_k1, Tensor cos_sin0, Tensor cos_sin1, SymInt batch_size, SymInt num_tokens0, SymInt num_tokens1, "
+          "SymInt num_heads_q, SymInt num_heads_k, SymInt head_size, bool is_interleaved, float eps) -> "
+          "(Tensor out_q01, Tensor out_k01)");
+    m.impl("fused_rope_rms_2way", c10::DispatchKey::CUDA, &fused_rope_rms_2way);
+    m.impl("fused_rope_rms_2way", c10::DispatchKey::Meta, &fused_rope_rms_2way_meta);
 
     // additive: amax divisor / clamp bound of the fp8 modes of allreduce_rms (448 OCP default, 240 reference)
     m.def("set_fp8_max(float value) -> ()");

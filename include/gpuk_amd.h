@@ -124,6 +124,26 @@ int gpuk_rope_rms_set_kv(const void *qkv, const void *qw, const void *kw, const 
                          float k_scale, float v_scale, int kv_dtype, void *stream);
 
 /*
+ * Two token streams (e.g. text and image) with their own norm weights and per-token cos/sin rows: per-head RMSNorm
+ * and rotation of q0/k0 with cos_sin0 and of q1/k1 with cos_sin1, outputs concatenated along the token axis.
+ *
+ * Stands behind fused_rope_rms_2way (src/ops/fused_rope.cpp:168-227 -> src/impl/rope_rms_impl.h:612-857).
+ * Rounding follows test/test_fused_rope_rms_2way.py:37-81.
+ *
+ *   q0, q1          : [batch, num_tokens{0,1}, num_heads_q, head_size] contiguous `dtype`, 16-byte aligned
+ *   k0, k1          : [batch, num_tokens{0,1}, num_heads_k, head_size]
+ *   w_q0 .. w_k1    : [head_size]
+ *   cos_sin0, 1     : [num_tokens{0,1}, head_size]; row t = cos | sin for token t of that stream
+ *   out_q01, out_k01: [batch, num_tokens0 + num_tokens1, num_heads_{q,k}, head_size]; stream 0 first
+ *   is_interleaved  : 1 rotates adjacent pairs (GPT-J style), 0 pairs element i with i + head_size/2 (NeoX style)
+ */
+int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1, const void *k1, const void *w_q0,
+                       const void *w_k0, const void *w_q1, const void *w_k1, const void *cos_sin0,
+                       const void *cos_sin1, int64_t batch_size, int64_t num_tokens0, int64_t num_tokens1,
+                       int64_t num_heads_q, int64_t num_heads_k, int64_t head_size, int is_interleaved, float eps,
+                       int dtype, void *out_q01, void *out_k01, void *stream);
+
+/*
  * Roofline calibration: dst[0..nbytes) = src[0..nbytes) with a plain streaming copy kernel (nbytes a
  * multiple of 16, both pointers 16-byte aligned).  Moves exactly 2*nbytes of HBM traffic; used to measure
  * the practical bandwidth ceiling and to scale the profiler's FETCH_SIZE / WRITE_SIZE readings.

@@ -60,6 +60,11 @@ def test_argument_validation_needs_no_gpu():
     assert s(p, p, p, p, p, 0, 1, 1, 4, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, p, p, p, p, 1.0, 1.0, 5, None) == 2  # kv dtype
     assert s(p, p, p, p, p, 0, 1, 1, 4, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, p, p, p, p, 0.0, 1.0, 1, None) == 1  # fp8 scale
     assert s(p, p, p, p, p, 0, 1, 1, 4, 2, 2, 2, 128, 1, None, 0, 1e-6, 0, None, p, p, p, 1.0, 1.0, 0, None) == 1
+    w = L.gpuk_rope_rms_2way
+    assert w(p, p, p, p, p, p, p, p, p, p, 1, 2, 2, 2, 2, 96, 0, 1e-6, 0, p, p, None) == 2     # head size
+    assert w(p, p, p, p, p, p, p, p, p, p, 1, -2, 2, 2, 2, 128, 0, 1e-6, 0, p, p, None) == 1   # negative tokens
+    assert w(p, p, p, p, p, p, p, p, p, p, 1, 2, 2, 2, 2, 128, 0, 1e-6, 0, None, p, None) == 1  # missing output
+    assert w(p, p, p, p, p, p, p, p, p, p, 0, 2, 2, 2, 2, 128, 0, 1e-6, 0, p, p, None) == 0    # empty batch
     assert L.gpuk_copy_bytes(p, p, 24, None) == 1 and L.gpuk_copy_bytes(p, p, 0, None) == 0
     assert L.gpuk_set_tuning(b"no_such_knob", 1) == 1 and L.gpuk_set_tuning(b"norm_quant_nchunk", 3) == 1
     assert L.gpuk_set_tuning(b"norm_quant_nchunk", 0) == 0
@@ -82,9 +87,23 @@ def test_torch_library_registers_reference_schemas():
     assert schema("fused_mrope_3d_rms_set_kv").endswith(
         "float eps, Tensor q, Tensor k_cache, Tensor v_cache, Tensor kv_loc, float k_scale, float v_scale) -> ()")
     for name in ("allreduce_rms", "fused_rope_rms", "fused_mrope_3d_rms", "fused_mrope_3d_rms_set_kv",
-                 "fused_rope_rms_set_kv", "set_fp8_max", "get_fp8_max"):
+                 "fused_rope_rms_2way", "fused_rope_rms_set_kv", "set_fp8_max", "get_fp8_max"):
         assert hasattr(gpuk, name)
     assert gpuk.fp8 == torch.float8_e4m3fn and gpuk.fp8_max_val == 448 and gpuk.fp8_policy_id == 1
+
+
+def test_two_way_op_has_a_meta_kernel():
+    """Shape inference without a device, as the reference registers it (src/register.cpp:62-63)."""
+    import gpuk_amd as gpuk
+
+    m = lambda *s: torch.empty(*s, dtype=torch.bfloat16, device="meta")
+    B, T0, T1, Hq, Hk, D = 2, 5, 7, 3, 2, 64
+    q01, k01 = gpuk.fused_rope_rms_2way(m(B, T0, Hq, D), m(B, T0, Hk, D), m(B, T1, Hq, D), m(B, T1, Hk, D), m(D), m(D),
+                                        m(D), m(D), m(T0, D), m(T1, D), B, T0, T1, Hq, Hk, D, False, 1e-6)
+    assert q01.shape == (B, T0 + T1, Hq, D) and k01.shape == (B, T0 + T1, Hk, D)
+    assert q01.device.type == "meta" and q01.dtype == torch.bfloat16
+    assert str(torch.ops.gpuk.fused_rope_rms_2way.default._schema).endswith(
+        "SymInt head_size, bool is_interleaved, float eps) -> (Tensor out_q01, Tensor out_k01)")
 
 
 def test_fp8_max_setter_round_trip():
