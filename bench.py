@@ -76,6 +76,34 @@ def per_launch_ms(fn, iters):
     return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
 
 
+def graph_time_us(call, n_in_graph=20, replays=30):
+    """us per call with n_in_graph calls recorded into one HIP graph (call(i) must launch on the current stream and
+    allocate nothing): the GPU-side cost of a call without the host's per-launch overhead."""
+    import torch
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(n_in_graph):
+            call(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(n_in_graph):
+            call(i)
+    for _ in range(3):
+        g.replay()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(replays):
+        g.replay()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) * 1e3 / (replays * n_in_graph)
+
+
 def traffic_from_profile(name):
     """HBM bytes per launch measured with rocprofv3 counters, if a summary for this workload is committed."""
     path = os.path.join(ROOT, "profiles", name)
@@ -218,16 +246,37 @@ def main():
                             "frac_of_8TBps": round(nbytes / (burst * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                             "algorithmic_bytes": nbytes}
 
+        # decode shapes: per call, eager (host launch overhead included) and replayed from a HIP graph of 20 calls on
+        # 20 distinct buffer sets (GPU-side cost)
         decode = {}
+        NG = 20
         for t in workloads.DECODE_TOKENS:
             d = workloads.config5_norm(t)
-            x, r_, g = d.x.to(dev), d.residual.to(dev), d.gamma.to(dev)
-            ro = torch.empty_like(x)
-            codes = torch.empty((t, 7168), dtype=torch.float8_e4m3fn, device=dev)
-            sc = torch.empty((t, 1), dtype=torch.float32, device=dev)
-            a_ms = event_time_ms(lambda i=0: capi.add_rmsnorm_quant(x, r_, g, ro, codes, sc, d.eps, 1), 300)
-            nbytes, avg, med, mn, burst = rope_case(workloads.config5_rope(t), 2)
-            decode[str(t)] = {"add_rmsnorm_quant_us": round(a_ms * 1e3, 2), "rope_kv_fp8_us": round(burst * 1e3, 2)}
+            g_ = d.gamma.to(dev)
+            nq = [(d.x.to(dev).clone(), d.residual.to(dev).clone(), torch.empty((t, 7168), dtype=torch.bfloat16, device=dev),
+                   torch.empty((t, 7168), dtype=torch.float8_e4m3fn, device=dev),
+                   torch.empty((t, 1), dtype=torch.float32, device=dev)) for _ in range(NG)]
+
+            def nq_call(i=0):
+                x, r_, ro, codes, sc = nq[i % NG]
+                capi.add_rmsnorm_quant(x, r_, g_, ro, codes, sc, d.eps, 1)
+
+            r = workloads.config5_rope(t)
+            k0, v0 = r.new_cache()
+            qw, kw, cs, pos, loc = (z.to(dev) for z in (r.qw, r.kw, r.cos_sin, r.positions, r.kv_loc))
+            kc, vc = k0.to(dev), v0.to(dev)
+            rp = [(r.qkv.to(dev).clone(), torch.empty((t, r.num_heads_q, r.head_size), dtype=torch.bfloat16, device=dev))
+                  for _ in range(NG)]
+
+            def rope_call(i=0):
+                qkv, q_out = rp[i % NG]
+                capi.rope_rms_set_kv(qkv, qw, kw, cs, pos, t, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
+                                     r.is_neox, r.eps, q_out, kc, vc, loc, r.k_scale, r.v_scale)
+
+            decode[str(t)] = {"add_rmsnorm_quant_us": round(graph_time_us(nq_call, NG), 2),
+                              "rope_kv_fp8_us": round(graph_time_us(rope_call, NG), 2),
+                              "add_rmsnorm_quant_eager_us": round(event_time_ms(nq_call, 200) * 1e3, 2),
+                              "rope_kv_fp8_eager_us": round(event_time_ms(rope_call, 200) * 1e3, 2)}
         extras["decode_us_per_call"] = decode
 
     out = {
