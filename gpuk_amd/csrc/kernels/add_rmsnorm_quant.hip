@@ -116,6 +116,7 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
 
     // ---- phase 2: n2 = rT(gamma * rT(res * rstd)); row amax for the dynamic scale
     float amax[ROWS];
+    float nv[ROWS][QUANT == GPUK_QUANT_NONE ? 1 : NCHUNK][8];
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
         // mean = sumsq / H as an exact IEEE quotient: by the reciprocal of H (computed on the host) while that is
@@ -123,18 +124,39 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
         const float mean = (sumsq[r] >= 0x1p-60f && sumsq[r] <= 0x1p100f) ? div_by_rcp(sumsq[r], hidden_f, rcp_hidden)
                                                                          : sumsq[r] / hidden_f;
         const float rstd = 1.0f / sqrtf(mean + eps);
-        uint32_t amax_bits = 0;
+        if constexpr (QUANT == GPUK_QUANT_NONE) {
 #pragma unroll
-        for (int i = 0; i < NCHUNK; ++i) {
+            for (int i = 0; i < NCHUNK; ++i) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t n1 = P::pack(P::lo(xv[r][i][j]) * rstd, P::hi(xv[r][i][j]) * rstd);
-                const uint32_t n2 = P::pack(P::lo(gv[i][j]) * P::lo(n1), P::hi(gv[i][j]) * P::hi(n1));
-                xv[r][i][j] = n2;  // xv now holds the normed row
-                if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) amax_bits = absmax_packed(amax_bits, n2);
+                for (int j = 0; j < 4; ++j) {
+                    const float lo = P::lo(gv[i][j]) * P::round(P::lo(xv[r][i][j]) * rstd);
+                    const float hi = P::hi(gv[i][j]) * P::round(P::hi(xv[r][i][j]) * rstd);
+                    xv[r][i][j] = P::pack(lo, hi);  // xv now holds the normed row
+                }
             }
+            amax[r] = 0.f;
+        } else {
+            // the normed row stays in fp32 registers, every value already rounded to the 16-bit type
+            // fmax drops NaNs where the reference's amax propagates them: they are tracked apart
+            float m0 = 0.f, m1 = 0.f;
+            bool any_nan = false;
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float lo = P::round(P::lo(gv[i][j]) * P::round(P::lo(xv[r][i][j]) * rstd));
+                    const float hi = P::round(P::hi(gv[i][j]) * P::round(P::hi(xv[r][i][j]) * rstd));
+                    nv[r][i][2 * j] = lo;
+                    nv[r][i][2 * j + 1] = hi;
+                    if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
+                        if (j & 1) m1 = __builtin_fmaxf(m1, __builtin_fmaxf(__builtin_fabsf(lo), __builtin_fabsf(hi)));
+                        else m0 = __builtin_fmaxf(m0, __builtin_fmaxf(__builtin_fabsf(lo), __builtin_fabsf(hi)));
+                        any_nan |= __builtin_isunordered(lo, hi);
+                    }
+                }
+            }
+            amax[r] = any_nan ? __builtin_nanf("") : __builtin_fmaxf(m0, m1);
         }
-        amax[r] = absmax_to_float<T>(amax_bits);
     }
 
     if constexpr (QUANT == GPUK_QUANT_NONE) {
@@ -164,16 +186,12 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
             uint8_t *out = reinterpret_cast<uint8_t *>(norm_out) + row_base[r] * 8;
             if (__builtin_expect(scale_in_fast_range(scale), 1)) {
                 const float rcp = 1.0f / scale;
-                auto encode = [&](const u32x4 &v) {
+                auto encode = [&](const float (&v)[8]) {
                     float q[8];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        q[2 * j] = div_by_rcp(P::lo(v[j]), scale, rcp);
-                        q[2 * j + 1] = div_by_rcp(P::hi(v[j]), scale, rcp);
-                        if constexpr (kClamp) {
-                            q[2 * j] = clamp_sym(q[2 * j], fp8_max);
-                            q[2 * j + 1] = clamp_sym(q[2 * j + 1], fp8_max);
-                        }
+                    for (int j = 0; j < 8; ++j) {
+                        q[j] = div_by_rcp(v[j], scale, rcp);
+                        if constexpr (kClamp) q[j] = clamp_sym(q[j], fp8_max);
                     }
                     return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
                 };
@@ -181,7 +199,7 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
                     const bool odd = tid & 1;
 #pragma unroll
                     for (int i = 0; i < NCHUNK; i += 2) {
-                        const u32x2 c0 = encode(xv[r][i]), c1 = encode(xv[r][i + 1]);
+                        const u32x2 c0 = encode(nv[r][i]), c1 = encode(nv[r][i + 1]);
                         // the even lane keeps iteration i and sends i+1; the odd lane the other way round
                         const u32x2 keep = odd ? c1 : c0, send = odd ? c0 : c1;
                         const u32x2 recv = {dpp_xor1_u32(send[0]), dpp_xor1_u32(send[1])};
@@ -193,7 +211,7 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
                 } else {
 #pragma unroll
                     for (int i = 0; i < NCHUNK; ++i) {
-                        const u32x2 codes = encode(xv[r][i]);
+                        const u32x2 codes = encode(nv[r][i]);
                         if (live[i] && row_ok[r]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
                     }
                 }
@@ -204,10 +222,7 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
                 for (int i = 0; i < NCHUNK; ++i) {
                     float q[8];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        q[2 * j] = clamp_sym(P::lo(xv[r][i][j]) / scale, fp8_max);
-                        q[2 * j + 1] = clamp_sym(P::hi(xv[r][i][j]) / scale, fp8_max);
-                    }
+                    for (int j = 0; j < 8; ++j) q[j] = clamp_sym(nv[r][i][j] / scale, fp8_max);
                     const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
                     if (live[i] && row_ok[r]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
                 }
@@ -269,8 +284,8 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
                 const u32x4 v = normed(c);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    amax = __builtin_fmaxf(amax, __builtin_fabsf(P::lo(v[j])));
-                    amax = __builtin_fmaxf(amax, __builtin_fabsf(P::hi(v[j])));
+                    amax = MaxOp::apply(amax, __builtin_fabsf(P::lo(v[j])));  // keeps a NaN, like the reference's amax
+                    amax = MaxOp::apply(amax, __builtin_fabsf(P::hi(v[j])));
                 }
             }
             float am[1] = {amax};

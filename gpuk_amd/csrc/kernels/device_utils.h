@@ -31,6 +31,9 @@ template <> struct Pack16<BF16> {
         f32x2 v = {a, b};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
     }
+    // rT(a) as a float: the high half of a pair whose low half is zero is the float's own bit pattern, so one
+    // conversion instruction rounds without a separate unpack
+    static __device__ __forceinline__ float round(float a) { return __builtin_bit_cast(float, pack(0.0f, a)); }
     // acc + lo(w)^2 + hi(w)^2 in one v_dot2c_f32_bf16 (products exact, fp32 accumulate)
     static __device__ __forceinline__ float add_squares(uint32_t w, float acc) {
         const bf16x2_t v = __builtin_bit_cast(bf16x2_t, w);
@@ -51,6 +54,7 @@ template <> struct Pack16<FP16> {
         const uint32_t h = __builtin_bit_cast(uint16_t, (_Float16)b);
         return l | (h << 16);
     }
+    static __device__ __forceinline__ float round(float a) { return (float)(_Float16)a; }
     static __device__ __forceinline__ float add_squares(uint32_t w, float acc) {
         const float a = lo(w), b = hi(w);
         return __builtin_fmaf(b, b, __builtin_fmaf(a, a, acc));
@@ -94,8 +98,12 @@ struct SumOp {
     static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
     static __device__ __forceinline__ float identity() { return 0.f; }
 };
-struct MaxOp {  // used on magnitudes only, so 0 is the identity
-    static __device__ __forceinline__ float apply(float a, float b) { return __builtin_fmaxf(a, b); }
+struct MaxOp {  // used on magnitudes only, so 0 is the identity.  Compared as bit patterns: for non-negative floats
+                // these order like the values, and a (positive) NaN beats everything, as in the reference's amax
+    static __device__ __forceinline__ float apply(float a, float b) {
+        const uint32_t x = __builtin_bit_cast(uint32_t, a), y = __builtin_bit_cast(uint32_t, b);
+        return __builtin_bit_cast(float, x > y ? x : y);
+    }
     static __device__ __forceinline__ float identity() { return 0.f; }
 };
 
@@ -156,17 +164,21 @@ __device__ __forceinline__ uint32_t cvt4_e4m3fn(float a, float b, float c, float
     return (uint32_t)w;
 }
 
+// clamp to [-bound, bound]; a NaN stays a NaN (v_med3_f32 alone would turn it into one of the bounds)
 __device__ __forceinline__ float clamp_sym(float v, float bound) {
-    return __builtin_amdgcn_fmed3f(v, -bound, bound);
+    const float c = __builtin_amdgcn_fmed3f(v, -bound, bound);
+    return v != v ? v : c;
 }
 
 // Correctly rounded fp32 quotient a/b given rcp = RN(1/b): one multiply and two fused
 // multiply-adds (Markstein's correction step).  Valid while a/b, the residual and rcp stay in the
-// normal range; callers guard the range of b once per row and fall back to `/` outside it.
+// normal range and b > 0; callers guard the range of b once per row and fall back to `/` outside it.
+// The correction step alone turns a quotient of -0 into +0 and an infinite one into NaN; v_div_fixup_f32 puts
+// back the sign and the zero / infinity / NaN a division gives for such numerators.
 __device__ __forceinline__ float div_by_rcp(float a, float b, float rcp) {
     float q = a * rcp;
     float e = __builtin_fmaf(-q, b, a);
-    return __builtin_fmaf(e, rcp, q);
+    return __builtin_amdgcn_div_fixupf(__builtin_fmaf(e, rcp, q), b, a);
 }
 
 }  // namespace gpuk

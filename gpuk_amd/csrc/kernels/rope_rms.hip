@@ -101,39 +101,36 @@ __device__ __forceinline__ void norm_rotate(const u32x4 &xa, const u32x4 &xb, co
     const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
     const float rstd = 1.0f / sqrtf(sumsq * (1.0f / D) + eps);  // D is a power of two: the product is exact
 
-    u32x4 na, nb;
+    // normed values stay in fp32 registers, each already rounded to the 16-bit type
+    float na[8], nb[8];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const uint32_t ta = P::pack(P::lo(xa[j]) * rstd, P::hi(xa[j]) * rstd);
-        const uint32_t tb = P::pack(P::lo(xb[j]) * rstd, P::hi(xb[j]) * rstd);
-        na[j] = P::pack(P::lo(wa[j]) * P::lo(ta), P::hi(wa[j]) * P::hi(ta));
-        nb[j] = P::pack(P::lo(wb[j]) * P::lo(tb), P::hi(wb[j]) * P::hi(tb));
+        na[2 * j] = P::round(P::lo(wa[j]) * P::round(P::lo(xa[j]) * rstd));
+        na[2 * j + 1] = P::round(P::hi(wa[j]) * P::round(P::hi(xa[j]) * rstd));
+        nb[2 * j] = P::round(P::lo(wb[j]) * P::round(P::lo(xb[j]) * rstd));
+        nb[2 * j + 1] = P::round(P::hi(wb[j]) * P::round(P::hi(xb[j]) * rstd));
     }
 
     if constexpr (NEOX) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float x1l = P::lo(na[j]), x1h = P::hi(na[j]), x2l = P::lo(nb[j]), x2h = P::hi(nb[j]);
+            const float x1l = na[2 * j], x1h = na[2 * j + 1], x2l = nb[2 * j], x2h = nb[2 * j + 1];
             const float cl = P::lo(cosv[j]), ch = P::hi(cosv[j]), sl = P::lo(sinv[j]), sh = P::hi(sinv[j]);
-            const uint32_t t1 = P::pack(x1l * cl, x1h * ch), t2 = P::pack(x2l * sl, x2h * sh);
-            const uint32_t t3 = P::pack(x2l * cl, x2h * ch), t4 = P::pack(x1l * sl, x1h * sh);
-            oa[j] = P::pack(P::lo(t1) - P::lo(t2), P::hi(t1) - P::hi(t2));
-            ob[j] = P::pack(P::lo(t3) + P::lo(t4), P::hi(t3) + P::hi(t4));
+            oa[j] = P::pack(P::round(x1l * cl) - P::round(x2l * sl), P::round(x1h * ch) - P::round(x2h * sh));
+            ob[j] = P::pack(P::round(x2l * cl) + P::round(x1l * sl), P::round(x2h * ch) + P::round(x1h * sh));
         }
     } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             {
-                const float x1 = P::lo(na[e]), x2 = P::hi(na[e]);
+                const float x1 = na[2 * e], x2 = na[2 * e + 1];
                 const float c = elem<T>(cosv, e), s = elem<T>(sinv, e);
-                const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
-                oa[e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
+                oa[e] = P::pack(P::round(x1 * c) - P::round(x2 * s), P::round(x2 * c) + P::round(x1 * s));
             }
             {
-                const float x1 = P::lo(nb[e]), x2 = P::hi(nb[e]);
+                const float x1 = nb[2 * e], x2 = nb[2 * e + 1];
                 const float c = elem<T>(cosv, 4 + e), s = elem<T>(sinv, 4 + e);
-                const uint32_t tc = P::pack(x1 * c, x2 * c), ts = P::pack(x2 * s, x1 * s);
-                ob[e] = P::pack(P::lo(tc) - P::lo(ts), P::hi(tc) + P::hi(ts));
+                ob[e] = P::pack(P::round(x1 * c) - P::round(x2 * s), P::round(x2 * c) + P::round(x1 * s));
             }
         }
     }
@@ -145,7 +142,7 @@ struct UnitState {
     uint32_t t, u;
     int head;
     bool live, active, is_q;
-    int64_t slot;
+    int64_t slot, p0, p1, p2;
     const uint16_t *token_in;
     u32x4 xa, xb, wa, wb, cosv, sinv, vchunk;
 };
@@ -194,14 +191,24 @@ struct RopeUnit {
         st.wa = *reinterpret_cast<const u32x4 *>(wsrc + c0(sub));
         st.wb = *reinterpret_cast<const u32x4 *>(wsrc + c1(sub));
 
+        st.p0 = a.positions[(int64_t)st.t * a.ps_token];
+        if constexpr (AXES == 3) {
+            st.p1 = a.positions[a.ps_axis + (int64_t)st.t * a.ps_token];
+            st.p2 = a.positions[2 * a.ps_axis + (int64_t)st.t * a.ps_token];
+        }
+    }
+
+    // The cos/sin loads, whose addresses wait for the positions.
+    static __device__ __forceinline__ void issue_table_loads(const RopeArgs &a, int lane, UnitState &st) {
+        if (!st.live) return;
+        const int sub = lane % LPH;
         const int fc = 8 * sub;
         const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin);
-        const int64_t p0 = a.positions[(int64_t)st.t * a.ps_token];
+        const int64_t p0 = st.p0;
         st.cosv = *reinterpret_cast<const u32x4 *>(table + p0 * D + fc);
         st.sinv = *reinterpret_cast<const u32x4 *>(table + p0 * D + HALF + fc);
         if constexpr (AXES == 3) {
-            const int64_t p1 = a.positions[a.ps_axis + (int64_t)st.t * a.ps_token];
-            const int64_t p2 = a.positions[2 * a.ps_axis + (int64_t)st.t * a.ps_token];
+            const int64_t p1 = st.p1, p2 = st.p2;
             if (p1 != p0 || p2 != p0) {  // wave-uniform; text tokens carry three equal positions
                 const u32x4 cos1 = *reinterpret_cast<const u32x4 *>(table + p1 * D + fc);
                 const u32x4 sin1 = *reinterpret_cast<const u32x4 *>(table + p1 * D + HALF + fc);
@@ -277,22 +284,20 @@ struct RopeUnit {
     }
 };
 
-// UPW: units per wave.  With 2, a wave has the loads of two units in flight before it starts on the first.
-template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8, int UPW>
+template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 __global__ void __launch_bounds__(512) rope_rms_kernel(const RopeArgs a) {
     using Unit = RopeUnit<T, D, NEOX, AXES, SETKV, KVFP8>;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t unit0 = (blockIdx.x * (blockDim.x >> 6) + wave) * UPW;
-    if (unit0 >= a.total_units) return;
+    const uint32_t unit = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (unit >= a.total_units) return;
     const int lane = threadIdx.x & 63;
-    UnitState st[UPW];
-#pragma unroll
-    for (int i = 0; i < UPW; ++i) Unit::issue_loads(a, unit0 + i, lane, st[i]);
+    UnitState st;
+    Unit::issue_loads(a, unit, lane, st);
+    Unit::issue_table_loads(a, lane, st);
     // Every load of the wave is in flight before the first use of any of them: without this fence the scheduler
     // moves arithmetic above later loads and the wave pays several memory round trips in a row.
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < UPW; ++i) Unit::finish(a, lane, st[i]);
+    Unit::finish(a, lane, st);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -377,18 +382,13 @@ int launch_2way_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned ba
 }
 
 int g_block_threads = 0;    // 0 = default
-int g_units_per_wave = 0;   // 0 = heuristic, else 1 or 2
 
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 int launch_one(const RopeArgs &a, hipStream_t stream) {
     const int threads = g_block_threads ? g_block_threads : 256;
-    const int upw = g_units_per_wave ? g_units_per_wave : 1;
-    const uint32_t units_per_block = threads / 64 * upw;
+    const uint32_t units_per_block = threads / 64;
     const uint32_t blocks = (a.total_units + units_per_block - 1) / units_per_block;
-    if (upw == 2)
-        rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8, 2><<<blocks, threads, 0, stream>>>(a);
-    else
-        rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8, 1><<<blocks, threads, 0, stream>>>(a);
+    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<blocks, threads, 0, stream>>>(a);
     return hip_status(hipGetLastError());
 }
 
@@ -503,7 +503,6 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
 
 void set_rope_tuning(int key, int value) {
     if (key == 0) g_block_threads = value;
-    if (key == 1) g_units_per_wave = value;
 }
 
 }  // namespace gpuk

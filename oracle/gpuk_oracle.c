@@ -331,7 +331,8 @@ int gpuk_oracle_rope_rms_2way(const uint16_t *q0, const uint16_t *k0, const uint
 }
 
 /* Model of the device's reciprocal-based quotient (one multiply, two fused multiply-adds with
- * rcp = RN(1/b)) against the IEEE quotient a/b: returns how many of the n pairs differ.  Lets the CPU
+ * rcp = RN(1/b), then the device's fix-up step, which restores the sign and hands zero, infinite and NaN
+ * numerators the result a division gives them) against the IEEE quotient a/b, for finite b > 0: returns how many of the n pairs differ.  Lets the CPU
  * tests show that the shortcut the HIP kernels take is exact on the operand ranges they guard. */
 int64_t gpuk_oracle_count_div_rcp_mismatch(const float *a, const float *b, int64_t n) {
     int64_t bad = 0;
@@ -340,6 +341,8 @@ int64_t gpuk_oracle_count_div_rcp_mismatch(const float *a, const float *b, int64
         float q = a[i] * rcp;
         float e = fmaf(-q, b[i], a[i]);
         float q1 = fmaf(e, rcp, q);
+        if (a[i] != a[i] || isinf(a[i]) || a[i] == 0.0f) q1 = a[i];  /* NaN, +-inf, +-0 pass through (b > 0) */
+        else q1 = copysignf(q1, a[i]);
         float want = a[i] / b[i];
         if (f32_bits(q1) != f32_bits(want) && !(q1 != q1 && want != want)) ++bad;
     }

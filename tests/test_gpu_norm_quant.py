@@ -60,6 +60,66 @@ def test_shapes_against_oracle(device, tokens, hidden, quant):
     check(inp, quant, got, static_scale=static, tag=f"[{tokens}x{hidden} q{quant}]")
 
 
+@pytest.mark.parametrize("hidden", [64, 4096, 8192, 65536 + 64])
+def test_non_finite_rows(device, hidden):
+    """NaN, infinities, overflowing squares and all-zero rows follow the oracle: a NaN anywhere in a row makes the
+    row's dynamic scale and all of its codes NaN (amax propagates it), an infinity zeroes the rest of its row
+    (rstd = 0) and leaves one NaN, squares that overflow give an all-zero row with scale 1, and a NaN in gamma
+    poisons that column (static) or every row's scale (dynamic)."""
+    print(f"case non-finite hidden={hidden}", flush=True)
+    inp = workloads.norm_quant_inputs(7, hidden, seed=hidden + 5, res_sigma=1.0, outlier_frac=0.0)
+    x, r = inp.x, inp.residual
+    x[0, 5] = float("nan")
+    x[1, hidden - 1] = float("inf")
+    x[2, :] = 3e38
+    r[2, :] = 0
+    x[3, :] = 0
+    r[3, :] = 0
+    x[4, 9] = -float("inf")
+    r[5, hidden // 2] = float("nan")
+
+    def same(got, want, is_fp8, what):
+        if is_fp8:
+            g8, w8 = got.cpu().view(torch.uint8), want.view(torch.uint8)
+            gn, wn = (g8 & 0x7F) == 0x7F, (w8 & 0x7F) == 0x7F
+            assert torch.equal(gn, wn), f"{what}: NaN codes in different places"
+            assert torch.equal(g8[~gn], w8[~wn]), f"{what}: finite codes differ"
+        else:
+            gf, wf = got.cpu().float(), want.float()
+            assert torch.equal(gf.isnan(), wf.isnan()), f"{what}: NaNs in different places"
+            keep = ~wf.isnan()
+            assert torch.equal(got.cpu().view(torch.int16)[keep], want.view(torch.int16)[keep]), f"{what}: values differ"
+
+    for gamma_nan in (False, True):
+        if gamma_nan:
+            inp.gamma[3] = float("nan")
+        for quant in (0, 1, 3):
+            static = torch.tensor([0.01]) if quant == 3 else None
+            res_ref, norm_ref, scale_ref = O.add_rmsnorm_quant_ref(x, r, inp.gamma, inp.eps, quant, static_scale=static)
+            res, norm, scale = run_capi(inp, quant, device, static_scale=static)
+            tag = f"[H={hidden} q{quant} gamma_nan={gamma_nan}]"
+            same(res, res_ref, False, tag + " residual_out")
+            if quant == 1:
+                sg, sw = scale.cpu().flatten(), scale_ref.flatten()
+                assert torch.equal(sg.isnan(), sw.isnan()), f"{tag}: NaN scales in different rows: {sg} vs {sw}"
+                assert_scales_close(sg[~sw.isnan()], sw[~sw.isnan()], tag + " finite scales")
+                # rows whose scale matches to the bit are compared code by code (row 6 is an ordinary row)
+                rows = [i for i in range(7) if sw[i].isnan() or sg[i] == sw[i]]
+                assert len(rows) >= 6
+                same(norm[rows], norm_ref[rows], True, tag + " codes")
+            elif quant == 3:
+                same(norm[:6], norm_ref[:6], True, tag + " codes")
+                g8, w8 = norm[6].cpu().view(torch.uint8), norm_ref[6].view(torch.uint8)
+                keep = (w8 & 0x7F) != 0x7F
+                assert torch.equal((g8 & 0x7F) != 0x7F, keep), f"{tag}: NaN codes of the ordinary row"
+                assert_codes_close(norm[6].cpu()[keep], norm_ref[6][keep], tag + " codes of the ordinary row")
+            else:
+                same(norm[:6], norm_ref[:6], False, tag + " norm_out")
+                keep = ~norm_ref[6].float().isnan()
+                assert torch.equal(~norm[6].cpu().float().isnan(), keep), f"{tag}: NaNs of the ordinary row"
+                assert_close_ulp16(norm[6].cpu()[keep], norm_ref[6][keep], tag + " norm_out of the ordinary row")
+
+
 @pytest.mark.parametrize("tokens,hidden", [(130, 520), (512, 7168), (256, 8192)])
 def test_rows_explained_by_rstd_ulp(device, tokens, hidden):
     """Every output row (normed values, scale and codes) is bit-identical to the oracle evaluated with

@@ -146,14 +146,31 @@ def test_rope_set_kv_head_mixes(device, hq, hk, hv, fp8):
     check_set_kv(inp, run_set_kv(inp, device), f"[set_kv {hq},{hk},{hv}]")
 
 
-@pytest.mark.parametrize("threads,units_per_wave", [(64, 1), (128, 2), (512, 1), (256, 2)])
-def test_launch_shape_variants(device, threads, units_per_wave):
-    """Workgroup size and units per wave are tuning choices only: every setting gives the same bits as the oracle."""
+ALIGNED_SECTIONS = {64: [8, 16, 8], 128: [16, 24, 24], 256: [48, 40, 40]}
+
+
+@pytest.mark.parametrize("neox", [True, False])
+@pytest.mark.parametrize("head_size", [64, 128, 256])
+def test_mrope_sections_on_multiples_of_8(device, neox, head_size):
+    """Chunked sections whose boundaries are multiples of 8: the 8 frequencies a lane owns then share one axis."""
+    print(f"case aligned sections neox={neox} D={head_size}", flush=True)
+    for fp8 in (False, True):
+        inp = make(131, 12, head_size, neox, seed=head_size + 7, mrope=True, interleaved=False, fp8=fp8, hk=4, hv=4)
+        inp.mrope_section = ALIGNED_SECTIONS[head_size]
+        check_set_kv(inp, run_set_kv(inp, device), f"[aligned D={head_size} fp8={fp8}]")
+        got = run_inplace(inp, device)
+        want = oracle_inplace(inp)
+        assert_rotated_close(got[:, :16], want[:, :16], "in place q,k")
+        assert_bits_equal(got[:, 16:], want[:, 16:], "in place v")
+
+
+@pytest.mark.parametrize("threads", [64, 128, 512])
+def test_launch_shape_variants(device, threads):
+    """The workgroup size is a tuning choice only: every setting gives the same bits as the oracle."""
     from gpuk_amd import capi
 
-    print(f"case variants threads={threads} units_per_wave={units_per_wave}", flush=True)
+    print(f"case variants threads={threads}", flush=True)
     capi.set_tuning("rope_block_threads", threads)
-    capi.set_tuning("rope_units_per_wave", units_per_wave)
     try:
         for hs, neox, mrope, fp8, heads in ((128, True, False, False, (32, 8, 8)), (64, False, True, True, (20, 20, 20)),
                                             (256, True, True, False, (9, 3, 3)), (128, False, False, True, (64, 8, 8))):
@@ -167,7 +184,6 @@ def test_launch_shape_variants(device, threads, units_per_wave):
             assert_bits_equal(got[:, nqk:], want[:, nqk:], "in place v")
     finally:
         capi.set_tuning("rope_block_threads", 0)
-        capi.set_tuning("rope_units_per_wave", 0)
 
 
 @pytest.mark.parametrize("hq,hk,hv,head_size", [(3, 1, 40, 64), (1, 1, 17, 256), (7, 2, 0, 128), (2, 9, 33, 128)])

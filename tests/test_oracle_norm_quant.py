@@ -179,4 +179,8 @@ def test_reciprocal_quotient_model_is_exact():
     b = torch.exp(torch.randn(2_000_000, generator=g) * 3).float()
     keep = (a / b).abs() >= 2 ** -12
     bad += c_oracle.count_div_rcp_mismatch(a[keep].contiguous(), b[keep].contiguous())
+    # zeros of either sign, infinities and NaN as numerators: the quotient keeps sign and class
+    special = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan")])
+    for s in (2.0 ** -60, 0.0123, 1.0, 2.0 ** 60):
+        bad += c_oracle.count_div_rcp_mismatch(special, torch.full_like(special, s))
     assert bad == 0
