@@ -40,6 +40,21 @@ fused_rope_rms_set_kv = torch.ops.gpuk.fused_rope_rms_set_kv       # additive: 1
 set_fp8_max = torch.ops.gpuk.set_fp8_max                           # additive
 get_fp8_max = torch.ops.gpuk.get_fp8_max                           # additive
 
+
+class _Traceable:
+    """The in-place operators under schemas that declare their writes (`Tensor(a!)`), each with a Meta kernel:
+    the overloads to call from code that goes through torch.compile / functionalisation.  Same arguments, same
+    kernels as the names above, whose schemas are the reference's and carry no alias annotations."""
+    allreduce_rms = torch.ops.gpuk.allreduce_rms.mut
+    fused_rope_rms = torch.ops.gpuk.fused_rope_rms.mut
+    fused_mrope_3d_rms = torch.ops.gpuk.fused_mrope_3d_rms.mut
+    fused_mrope_3d_rms_set_kv = torch.ops.gpuk.fused_mrope_3d_rms_set_kv.mut
+    fused_rope_rms_set_kv = torch.ops.gpuk.fused_rope_rms_set_kv.mut
+    fused_rope_rms_2way = torch.ops.gpuk.fused_rope_rms_2way.default   # functional already
+
+
+traceable = _Traceable
+
 # gfx950 encodes OCP e4m3fn.  The reference defaults to the MI300-only e4m3fnuz (gpuk/__init__.py:38)
 # and uses 240 as e4m3fn's maximum (:42-46); 448 is the OCP maximum.  `set_fp8_max(240)` restores the
 # reference's divisor (codes up to 240 are identical in both encodings).
@@ -96,11 +111,27 @@ class GPUKDistEnv:
 
     @contextmanager
     def capture(self):
+        """Wraps a stream capture (gpuk/__init__.py:112-120).  The fused op allocates nothing and launches on the
+        current stream, so at world size 1 a captured graph needs no pointer registration afterwards."""
         try:
             self._IS_CAPTURING = True
             yield
         finally:
             self._IS_CAPTURING = False
+            # consume_capture() synchronises the device, which is not allowed while the stream is still capturing
+            if not self.disabled and not torch.cuda.is_current_stream_capturing():
+                self.consume_capture()
+
+    def capture_(self, input: torch.Tensor):
+        """Per-call bookkeeping of the reference (gpuk/__init__.py:122-129): remember that a capture happened, and
+        after it ended do what consume_capture does."""
+        if torch.compiler.is_compiling():
+            return
+        if torch.cuda.is_current_stream_capturing():
+            self._IS_CAPTURED = True
+        elif self._IS_CAPTURED:
+            self.consume_capture()
+            self._IS_CAPTURED = False
 
     def allreduce_native(self, allreduce_in):
         return allreduce_in.clone()
@@ -108,11 +139,26 @@ class GPUKDistEnv:
     def allreduce(self, allreduce_in):
         return allreduce_in.clone()
 
+    def allreduce_add_rms_native(self, allreduce_in, residual_in, rms_weight, eps, fp8_out=False):
+        """The unfused torch sequence the reference keeps beside the fused op (gpuk/__init__.py:147-173), minus the
+        all-reduce: a handful of torch kernels on the tensors' device, for comparison and timing only."""
+        residual_out = allreduce_in + residual_in
+        variance = residual_out.float().pow(2).mean(-1, keepdim=True)
+        norm_out = rms_weight * (residual_out * torch.rsqrt(variance + eps)).to(residual_out.dtype)
+        if fp8_out:
+            limit = float(get_fp8_max())
+            scale = norm_out.float().abs().max(dim=-1, keepdim=True)[0] / limit
+            norm_out = (norm_out / scale).clamp_(min=-limit, max=limit).to(fp8)
+            return residual_out, norm_out, scale
+        scale_out = torch.empty(allreduce_in.shape[0], 1, dtype=torch.float32, device=allreduce_in.device)
+        return residual_out, norm_out, scale_out
+
     def allreduce_add_rms_fused(self, allreduce_in, residual_in, rms_weight, eps, fp8_out=False, static_scale=None):
         """gpuk/__init__.py:175-205.  Returns (residual_out, norm_out, scale_out).
 
         `static_scale` (additive): a 1-element fp32 tensor; selects per-tensor static quantisation.
         """
+        self.capture_(allreduce_in)
         residual_out = torch.empty_like(residual_in)
         if fp8_out:
             norm_out = torch.empty_like(allreduce_in, dtype=fp8)
@@ -126,5 +172,7 @@ class GPUKDistEnv:
             norm_out = torch.empty_like(allreduce_in)
             scale_out = torch.empty(1, dtype=torch.float32, device=allreduce_in.device)
             quant = QUANT_NONE
-        allreduce_rms(self.fptr, allreduce_in, residual_in, rms_weight, residual_out, norm_out, scale_out, eps, quant)
+        # the overload whose schema declares the three writes: same kernel, and the call survives tracing
+        traceable.allreduce_rms(self.fptr, allreduce_in, residual_in, rms_weight, residual_out, norm_out, scale_out,
+                                eps, quant)
         return residual_out, norm_out, scale_out

@@ -189,3 +189,43 @@ def test_bench_refuses_more_than_one_gpu():
 
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "single-GPU" in r.stderr
+
+
+def test_mut_overloads_differ_from_reference_schemas_only_in_alias_annotations():
+    """Every in-place operator has an overload `.mut` whose schema, with the `(x!)` annotations removed, is the
+    reference's string (src/register.cpp:37-55), and which declares at least one written tensor."""
+    import re
+
+    import gpuk_amd  # noqa: F401  (loads the library)
+
+    for name in ("allreduce_rms", "fused_rope_rms", "fused_mrope_3d_rms", "fused_mrope_3d_rms_set_kv",
+                 "fused_rope_rms_set_kv"):
+        packet = getattr(torch.ops.gpuk, name)
+        assert packet.overloads() == ["default", "mut"], name
+        plain, annotated = str(packet.default._schema), str(packet.mut._schema)
+        assert "!)" in annotated and "!)" not in plain
+        assert re.sub(r"\([a-z]!\)", "", annotated).replace(name + ".mut(", name + "(") == plain
+    written = {a.name for a in torch.ops.gpuk.allreduce_rms.mut._schema.arguments if a.alias_info and a.alias_info.is_write}
+    assert written == {"residual_out", "norm_out", "scale_out"}
+    written = {a.name for a in torch.ops.gpuk.fused_mrope_3d_rms_set_kv.mut._schema.arguments
+               if a.alias_info and a.alias_info.is_write}
+    assert written == {"q", "k_cache", "v_cache"}
+    written = {a.name for a in torch.ops.gpuk.fused_rope_rms.mut._schema.arguments if a.alias_info and a.alias_info.is_write}
+    assert written == {"qkv"}
+
+
+def test_mut_overloads_have_meta_kernels():
+    """On meta tensors the `.mut` overloads run (and do nothing); the reference-schema overloads have no Meta
+    kernel and refuse, as in the reference."""
+    import gpuk_amd
+
+    x = torch.empty((4, 64), dtype=torch.bfloat16, device="meta")
+    g = torch.empty((64,), dtype=torch.bfloat16, device="meta")
+    codes = torch.empty((4, 64), dtype=torch.float8_e4m3fn, device="meta")
+    scale = torch.empty((4, 1), device="meta")
+    assert gpuk_amd.traceable.allreduce_rms(0, x, x, g, x, codes, scale, 1e-6, 1) is None
+    with pytest.raises(NotImplementedError):
+        gpuk_amd.allreduce_rms(0, x, x, g, x, codes, scale, 1e-6, 1)
+    qkv = torch.empty((4, 6, 64), dtype=torch.bfloat16, device="meta")
+    pos = torch.empty((4,), dtype=torch.int64, device="meta")
+    assert gpuk_amd.traceable.fused_rope_rms(qkv, g, g, x, pos, 4, 2, 2, 2, 64, True, 1e-6) is None
