@@ -278,6 +278,37 @@ def main():
                               "add_rmsnorm_quant_eager_us": round(event_time_ms(nq_call, 200) * 1e3, 2),
                               "rope_kv_fp8_eager_us": round(event_time_ms(rope_call, 200) * 1e3, 2)}
         extras["decode_us_per_call"] = decode
+        # the floor under those: a 1024-element increment kernel (one workgroup), same two ways of launching
+        small = [torch.zeros(1024, dtype=torch.float32, device=dev) for _ in range(NG)]
+
+        def small_call(i=0):
+            capi.increment_floats(small[i % NG], 1024)
+
+        extras["small_kernel_us_per_call"] = {"graph": round(graph_time_us(small_call, NG), 2),
+                                              "eager": round(event_time_ms(small_call, 200) * 1e3, 2)}
+
+        # a caller of both paths: one Qwen3-8B-sized decoder block, decode step of 32 sequences with 256 cached
+        # positions each, replayed from a HIP graph; fused operators against the torch sequence on the same weights
+        # (GEMMs and attention are torch's in both, so the difference is the memory-bound glue)
+        with torch.no_grad():
+            from gpuk_amd import consumer
+
+            bargs = consumer.BlockArgs()
+            torch.manual_seed(0)
+            block = consumer.TransformerBlock(bargs, dev)
+            nseq, ctx, bs = 32, 256, 16
+            per_seq = ctx // bs + 1
+            cache = consumer.PagedKVCache(nseq * per_seq, bs, bargs.n_kv_heads, bargs.head_dim, bargs.dtype, dev)
+            table = torch.randperm(nseq * per_seq, device=dev).view(nseq, per_seq)
+            idx = consumer.decode_batch(cache, table, torch.full((nseq,), ctx, device=dev))
+            hid = torch.randn((nseq, bargs.dim), device=dev).to(bargs.dtype)
+            res = torch.randn((nseq, bargs.dim), device=dev).to(bargs.dtype)
+            fused_us = graph_time_us(lambda i=0: block(hid, res, *idx[:2], cache, *idx[2:]), 4, 20)
+            unfused_us = graph_time_us(lambda i=0: block.forward_unfused(hid, res, *idx[:2], cache, *idx[2:]), 4, 20)
+            extras["decoder_block_decode_us"] = {"fused_ops": round(fused_us, 1), "torch_sequence": round(unfused_us, 1),
+                                                 "sequences": nseq, "context": ctx, "dim": bargs.dim,
+                                                 "heads": [bargs.n_heads, bargs.n_kv_heads, bargs.n_kv_heads]}
+            del block, cache
 
     out = {
         "metric": "HBM GB/s add+RMSNorm+FP8 per-token quant @8192x8192 bf16",

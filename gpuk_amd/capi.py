@@ -14,7 +14,7 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libgpuk_amd.so")
 
 EXPORTS = ("gpuk_status_string", "gpuk_abi_version", "gpuk_add_rmsnorm_quant", "gpuk_rope_rms",
-           "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_set_tuning")
+           "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_increment_floats", "gpuk_set_tuning")
 
 DTYPE = {torch.bfloat16: 0, torch.float16: 1}
 QUANT_NONE, QUANT_FP8_DYNAMIC, QUANT_FP8_E4M3FNUZ, QUANT_FP8_STATIC = 0, 1, 2, 3
@@ -53,6 +53,8 @@ def lib():
         L.gpuk_rope_rms_2way.restype = C.c_int
         L.gpuk_rope_rms_2way.argtypes = [C.c_void_p] * 10 + [C.c_int64] * 6 + [C.c_int, C.c_float, C.c_int,
                                                                              C.c_void_p, C.c_void_p, C.c_void_p]
+        L.gpuk_increment_floats.restype = C.c_int
+        L.gpuk_increment_floats.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
         L.gpuk_copy_bytes.restype = C.c_int
         L.gpuk_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
         _lib = L
@@ -117,6 +119,12 @@ def rope_rms_set_kv(qkv, qw, kw, cos_sin, positions, T, Hq, Hk, Hv, D, is_neox, 
                                     k_scale, v_scale, kv, _stream(stream))
     if rc:
         raise GpukError(rc, "gpuk_rope_rms_set_kv")
+
+
+def increment_floats(data, n: int, stream=None) -> None:
+    rc = lib().gpuk_increment_floats(_ptr(data), n, _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_increment_floats")
 
 
 def copy_bytes(dst, src, nbytes: int, stream=None) -> None:

@@ -151,8 +151,18 @@ int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1, const voi
  */
 int gpuk_copy_bytes(void *dst, const void *src, int64_t nbytes, void *stream);
 
-/* Development knob for sweeps: key "norm_quant_nchunk" (0 = heuristic, else 1/2/4/8 chunks per lane),
- * "rope_heads_per_wave" ... Unknown keys return GPUK_ERR_INVALID_ARG.  Not part of the reference. */
+/*
+ * Launch-cost calibration: data[i] += 1 for i in [0, n) (data 16-byte aligned).  With a small n the call costs
+ * what launching and draining any kernel costs, the floor under decode-sized calls.
+ * Counterpart of the reference's micro-benchmark test/cpp/test_small_kernel.cpp:85-126.
+ */
+int gpuk_increment_floats(float *data, int64_t n, void *stream);
+
+/* Launch-shape knobs for sweeps and for the tests that show the results do not depend on them; value 0 restores
+ * the built-in choice.  Keys: "norm_quant_nchunk" (1/2/4/8 16-byte chunks per lane), "norm_quant_threads" (lanes
+ * per row), "norm_quant_rows" (1 or 2 rows per workgroup), "norm_quant_paired_stores" (0/1), "norm_quant_lds_pad"
+ * (bytes of idle LDS per workgroup), "rope_block_threads" (64/128/256/512).  Unknown keys or values return
+ * GPUK_ERR_INVALID_ARG.  Not part of the reference. */
 int gpuk_set_tuning(const char *key, int value);
 
 #ifdef __cplusplus

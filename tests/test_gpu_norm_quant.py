@@ -306,3 +306,15 @@ def test_matches_torch_on_gpu(device):
     assert d_kernel.max().item() <= 1
     assert (d_kernel != 0).sum().item() <= 1.1 * (d_torch != 0).sum().item() + 16
     assert_scales_close(scale, s_gpu, "scale vs torch-GPU")
+
+
+def test_increment_floats_calibration_kernel(device):
+    """The launch-cost calibration kernel adds one to every element, tail included."""
+    from gpuk_amd import capi
+
+    for n in (0, 1, 3, 1024, 4099):
+        data = torch.arange(n + 4, dtype=torch.float32, device=device)
+        capi.increment_floats(data, n)
+        want = torch.arange(n + 4, dtype=torch.float32)
+        want[:n] += 1
+        assert torch.equal(data.cpu(), want), n
