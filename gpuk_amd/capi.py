@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "lib
 EXPORTS = ("gpuk_status_string", "gpuk_abi_version", "gpuk_add_rmsnorm_quant", "gpuk_rope_rms",
            "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_increment_floats", "gpuk_set_tuning")
 
-DTYPE = {torch.bfloat16: 0, torch.float16: 1}
+DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 QUANT_NONE, QUANT_FP8_DYNAMIC, QUANT_FP8_E4M3FNUZ, QUANT_FP8_STATIC = 0, 1, 2, 3
 KV_SAME, KV_E4M3FN = 0, 1
 

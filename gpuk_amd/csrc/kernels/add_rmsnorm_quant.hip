@@ -309,6 +309,67 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
     }
 }
 
+// fp32 activations: the reference dispatches them through the same template (src/ops/all_reduce_fusion.cpp:375-378).
+// A compatibility path, not a tuned one: three sweeps over the row like the long-row kernel, 4 elements per chunk.
+// Rounding to the activation type is the identity here, so the oracle's sequence is plain fp32 arithmetic:
+// res = x + r; n = gamma * (res * rstd); code = e4m3fn(clamp(n / scale)).
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int QUANT>
+__global__ void __launch_bounds__(kMaxThreads)
+add_rmsnorm_quant_f32_rows(const f32x4 *__restrict__ x, const f32x4 *__restrict__ residual_in,
+                           const f32x4 *__restrict__ gamma, f32x4 *residual_out, void *__restrict__ norm_out,
+                           float *__restrict__ scale_io, int chunks_per_row, float hidden_f, float eps, float fp8_max) {
+    __shared__ float s_sum[kReduceSlots];
+    __shared__ float s_max[kReduceSlots];
+    const int tid = threadIdx.x;
+    const int num_waves = blockDim.x >> 6;
+    const int64_t row_base = (int64_t)blockIdx.x * chunks_per_row;
+
+    float ss = 0.f;
+    for (int c = tid; c < chunks_per_row; c += blockDim.x) {
+        const f32x4 res = x[row_base + c] + residual_in[row_base + c];
+        residual_out[row_base + c] = res;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ss = __builtin_fmaf(res[j], res[j], ss);
+    }
+    float sumsq[1] = {ss};
+    block_allreduce<SumOp, 1>(sumsq, s_sum, num_waves);
+    const float rstd = 1.0f / sqrtf(sumsq[0] / hidden_f + eps);
+
+    auto normed = [&](int c) {
+        const f32x4 v = residual_out[row_base + c];  // written by this lane above
+        return gamma[c] * (v * rstd);
+    };
+
+    if constexpr (QUANT == GPUK_QUANT_NONE) {
+        f32x4 *out = reinterpret_cast<f32x4 *>(norm_out) + row_base;
+        for (int c = tid; c < chunks_per_row; c += blockDim.x) out[c] = normed(c);
+    } else {
+        float scale;
+        if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
+            float amax = 0.f;
+            for (int c = tid; c < chunks_per_row; c += blockDim.x) {
+                const f32x4 v = normed(c);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) amax = MaxOp::apply(amax, __builtin_fabsf(v[j]));
+            }
+            float am[1] = {amax};
+            block_allreduce<MaxOp, 1>(am, s_max, num_waves);
+            scale = am[0] == 0.f ? 1.f : am[0] / fp8_max;
+            if (tid == 0) scale_io[blockIdx.x] = scale;
+        } else {
+            scale = scale_io[0];
+        }
+        uint32_t *out = reinterpret_cast<uint32_t *>(norm_out) + row_base;
+        for (int c = tid; c < chunks_per_row; c += blockDim.x) {
+            const f32x4 v = normed(c);
+            out[c] = cvt4_e4m3fn(clamp_sym(v[0] / scale, fp8_max), clamp_sym(v[1] / scale, fp8_max),
+                                 clamp_sym(v[2] / scale, fp8_max), clamp_sym(v[3] / scale, fp8_max));
+        }
+    }
+}
+
 int g_force_nchunk = 0;   // 0 = heuristic; set through gpuk_set_tuning for sweeps
 int g_force_threads = 0;  // 0 = heuristic
 int g_rows = 0;           // rows per workgroup: 0 = heuristic, 1 or 2
@@ -381,6 +442,33 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
     return hip_status(hipGetLastError());
 }
 
+template <int QUANT>
+int launch_f32(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
+               float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream) {
+    const int chunks = (int)(hidden / 4);
+    const int want = (chunks + 63) / 64 * 64;
+    const int threads = want < kMaxThreads ? want : kMaxThreads;
+    add_rmsnorm_quant_f32_rows<QUANT><<<dim3((unsigned)tokens), threads, 0, stream>>>(
+        static_cast<const f32x4 *>(x), static_cast<const f32x4 *>(residual_in), static_cast<const f32x4 *>(gamma),
+        static_cast<f32x4 *>(residual_out), norm_out, scale, chunks, (float)hidden, eps, fp8_max);
+    return hip_status(hipGetLastError());
+}
+
+int launch_quant_f32(int quant_mode, const void *x, const void *residual_in, const void *gamma, void *residual_out,
+                     void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max,
+                     hipStream_t stream) {
+    switch (quant_mode) {
+        case GPUK_QUANT_NONE:
+            return launch_f32<GPUK_QUANT_NONE>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+        case GPUK_QUANT_FP8_DYNAMIC:
+            return launch_f32<GPUK_QUANT_FP8_DYNAMIC>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+        case GPUK_QUANT_FP8_STATIC:
+            return launch_f32<GPUK_QUANT_FP8_STATIC>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+        default:
+            return GPUK_ERR_UNSUPPORTED;
+    }
+}
+
 template <typename T>
 int launch_quant(int quant_mode, const void *x, const void *residual_in, const void *gamma, void *residual_out,
                  void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max,
@@ -429,6 +517,8 @@ extern "C" int gpuk_add_rmsnorm_quant(const void *x, const void *residual_in, co
             return launch_quant<BF16>(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
         case GPUK_DTYPE_FP16:
             return launch_quant<FP16>(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
+        case GPUK_DTYPE_F32:
+            return launch_quant_f32(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
         default:
             return GPUK_ERR_UNSUPPORTED;
     }

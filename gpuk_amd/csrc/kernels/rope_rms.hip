@@ -301,6 +301,101 @@ __global__ void __launch_bounds__(512) rope_rms_kernel(const RopeArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// fp32 activations: the reference dispatches them through the same templates (src/ops/fused_rope.cpp:27-30, :108-111).
+// A compatibility path, not a tuned one: one wave per (token, head), lane l owns rotation pairs l, l+64, ...;
+// with a KV cache the V heads get waves of their own that copy or quantise.  Rounding to the activation type is the
+// identity, so the oracle's sequence is plain fp32 arithmetic with every product rounded before the add.
+template <int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
+__global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
+    constexpr int HALF = D / 2;
+    constexpr int PPL = (HALF + 63) / 64;  // pairs per lane
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t unit = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (unit >= a.total_units) return;
+    const int lane = threadIdx.x & 63;
+    const uint32_t t = a.upt_magic ? __umulhi(unit, a.upt_magic) : unit;
+    const int h = (int)(unit - t * a.units_per_token);  // head index inside the token's qkv row
+    const int heads_qk = a.hq + a.hk, heads_all = heads_qk + a.hv;
+    const float *src = static_cast<const float *>(a.qkv_in) + ((int64_t)t * heads_all + h) * D;
+
+    if (h >= heads_qk) {  // a V head: only reached with a KV cache
+        if constexpr (SETKV) {
+            const int64_t row = (a.kv_loc[t] * a.hv + (h - heads_qk)) * D;
+            for (int e = lane; e < D; e += 64) {
+                const float v = src[e];
+                if constexpr (KVFP8) {
+                    static_cast<uint8_t *>(a.v_cache)[row + e] =
+                        (uint8_t)cvt4_e4m3fn(clamp_sym(v / a.v_scale, kE4M3Max), 0.f, 0.f, 0.f);
+                } else {
+                    static_cast<float *>(a.v_cache)[row + e] = v;
+                }
+            }
+        }
+        return;
+    }
+
+    const bool is_q = h < a.hq;
+    const float *w = static_cast<const float *>(is_q ? a.qw : a.kw);
+    float x1[PPL], x2[PPL];
+    int i1[PPL], i2[PPL];
+    bool live[PPL];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < PPL; ++k) {
+        const int p = lane + 64 * k;
+        live[k] = p < HALF;
+        const int pc = live[k] ? p : 0;
+        i1[k] = NEOX ? pc : 2 * pc;
+        i2[k] = NEOX ? pc + HALF : 2 * pc + 1;
+        x1[k] = live[k] ? src[i1[k]] : 0.f;
+        x2[k] = live[k] ? src[i2[k]] : 0.f;
+        ss = __builtin_fmaf(x1[k], x1[k], ss);
+        ss = __builtin_fmaf(x2[k], x2[k], ss);
+    }
+    ss = wave_allreduce<SumOp>(ss);
+    const float rstd = 1.0f / sqrtf(ss * (1.0f / D) + a.eps);
+
+    const float *table = static_cast<const float *>(a.cos_sin);
+    const int64_t p0 = a.positions[(int64_t)t * a.ps_token];
+    int64_t p1 = p0, p2 = p0;
+    if constexpr (AXES == 3) {
+        p1 = a.positions[a.ps_axis + (int64_t)t * a.ps_token];
+        p2 = a.positions[2 * a.ps_axis + (int64_t)t * a.ps_token];
+    }
+    float *dst;
+    uint8_t *dst8 = nullptr;
+    if constexpr (!SETKV) {
+        dst = static_cast<float *>(a.qkv_out) + ((int64_t)t * heads_all + h) * D;
+    } else if (is_q) {
+        dst = static_cast<float *>(a.q_out) + ((int64_t)t * a.hq + h) * D;
+    } else {
+        const int64_t row = (a.kv_loc[t] * a.hk + (h - a.hq)) * D;
+        dst = static_cast<float *>(a.k_cache) + row;          // used when the cache is fp32
+        dst8 = static_cast<uint8_t *>(a.k_cache) + row;       // used when it is fp8
+    }
+#pragma unroll
+    for (int k = 0; k < PPL; ++k) {
+        if (!live[k]) continue;
+        const int f = lane + 64 * k;  // rotary frequency of this pair
+        int64_t pos = p0;
+        if constexpr (AXES == 3) {
+            const bool on1 = (a.axis1[f >> 5] >> (f & 31)) & 1u, on2 = (a.axis2[f >> 5] >> (f & 31)) & 1u;
+            pos = on2 ? p2 : (on1 ? p1 : p0);
+        }
+        const float c = table[pos * D + f], s = table[pos * D + HALF + f];
+        const float n1 = w[i1[k]] * (x1[k] * rstd), n2 = w[i2[k]] * (x2[k] * rstd);
+        const float o1 = n1 * c - n2 * s, o2 = n2 * c + n1 * s;
+        if (SETKV && KVFP8 && !is_q) {
+            dst8[i1[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym(o1 / a.k_scale, kE4M3Max), 0.f, 0.f, 0.f);
+            dst8[i2[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym(o2 / a.k_scale, kE4M3Max), 0.f, 0.f, 0.f);
+        } else {
+            dst[i1[k]] = o1;
+            dst[i2[k]] = o2;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // Two token streams with their own norm weights and per-token cos/sin rows, outputs concatenated along the token
 // axis (reference: fused_rope_rms_2way, src/ops/fused_rope.cpp:168-227 -> src/impl/rope_rms_impl.h:612-857).
 // Per batch entry there are four segments of heads, each a contiguous [tokens, heads, D] block:
@@ -409,6 +504,35 @@ int launch_style(const RopeArgs &a, bool neox, int n_axes, bool set_kv, bool kv_
                        : launch_mode<T, D, false, 1>(a, set_kv, kv_fp8, stream);
 }
 
+template <int D, bool NEOX, int AXES>
+int launch_f32_mode(const RopeArgs &a, bool set_kv, bool kv_fp8, hipStream_t stream) {
+    const uint32_t blocks = (a.total_units + 3) / 4;
+    if (!set_kv) rope_rms_f32_kernel<D, NEOX, AXES, false, false><<<blocks, 256, 0, stream>>>(a);
+    else if (kv_fp8) rope_rms_f32_kernel<D, NEOX, AXES, true, true><<<blocks, 256, 0, stream>>>(a);
+    else rope_rms_f32_kernel<D, NEOX, AXES, true, false><<<blocks, 256, 0, stream>>>(a);
+    return hip_status(hipGetLastError());
+}
+
+template <int D>
+int launch_f32_style(const RopeArgs &a, bool neox, int n_axes, bool set_kv, bool kv_fp8, hipStream_t stream) {
+    if (neox) {
+        return n_axes == 3 ? launch_f32_mode<D, true, 3>(a, set_kv, kv_fp8, stream)
+                           : launch_f32_mode<D, true, 1>(a, set_kv, kv_fp8, stream);
+    }
+    return n_axes == 3 ? launch_f32_mode<D, false, 3>(a, set_kv, kv_fp8, stream)
+                       : launch_f32_mode<D, false, 1>(a, set_kv, kv_fp8, stream);
+}
+
+int launch_f32_head_size(const RopeArgs &a, int64_t head_size, bool neox, int n_axes, bool set_kv, bool kv_fp8,
+                         hipStream_t stream) {
+    switch (head_size) {
+        case 64: return launch_f32_style<64>(a, neox, n_axes, set_kv, kv_fp8, stream);
+        case 128: return launch_f32_style<128>(a, neox, n_axes, set_kv, kv_fp8, stream);
+        case 256: return launch_f32_style<256>(a, neox, n_axes, set_kv, kv_fp8, stream);
+        default: return GPUK_ERR_UNSUPPORTED;
+    }
+}
+
 template <typename T>
 int launch_head_size(const RopeArgs &a, int64_t head_size, bool neox, int n_axes, bool set_kv, bool kv_fp8,
                      hipStream_t stream) {
@@ -445,7 +569,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     if (T < 0 || hq < 0 || hk < 0 || hv < 0) return GPUK_ERR_INVALID_ARG;
     if (n_axes != 1 && n_axes != 3) return GPUK_ERR_INVALID_ARG;
     if (D != 64 && D != 128 && D != 256) return GPUK_ERR_UNSUPPORTED;
-    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16) return GPUK_ERR_UNSUPPORTED;
+    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32) return GPUK_ERR_UNSUPPORTED;
     if (set_kv && kv_dtype != GPUK_KV_SAME && kv_dtype != GPUK_KV_E4M3FN) return GPUK_ERR_UNSUPPORTED;
     if (hq > 0x7fffff || hk > 0x7fffff || hv > 0x7fffff) return GPUK_ERR_UNSUPPORTED;
     RopeArgs a{};
@@ -471,6 +595,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     int64_t upt = (hq + hk + hpw - 1) / hpw;
     if (upt == 0) upt = (hv * (D / 8) + 63) / 64;
     if (hq + hk == 0) return GPUK_ERR_UNSUPPORTED;  // a qkv row without Q and K heads has nothing to rotate
+    if (dtype == GPUK_DTYPE_F32) upt = hq + hk + (set_kv ? hv : 0);  // the fp32 path: one wave per head
     // mulhi(unit, ceil(2^32/upt)) equals unit / upt while unit * upt < 2^32
     if (upt * T >= 0x7fffffffLL || upt * T * upt >= (1LL << 32)) return GPUK_ERR_UNSUPPORTED;
     a.qkv_in = qkv_in;
@@ -495,6 +620,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     a.k_scale = k_scale;
     a.v_scale = v_scale;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == GPUK_DTYPE_F32) return launch_f32_head_size(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
     if (dtype == GPUK_DTYPE_BF16) return launch_head_size<BF16>(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
     return launch_head_size<FP16>(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
 }

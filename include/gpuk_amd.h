@@ -35,7 +35,8 @@ typedef enum gpuk_status {
  * src/ops/all_reduce_fusion.cpp:375, src/ops/fused_rope.cpp:27-31). */
 typedef enum gpuk_dtype {
     GPUK_DTYPE_BF16 = 0,
-    GPUK_DTYPE_FP16 = 1
+    GPUK_DTYPE_FP16 = 1,
+    GPUK_DTYPE_F32 = 2 /* compatibility path (the reference dispatches float too); not tuned like the 16-bit types */
 } gpuk_dtype;
 
 /* quant_type of the allreduce_rms op.  0/1/2 are the reference's QuantType
