@@ -162,7 +162,8 @@ int gpuk_increment_floats(float *data, int64_t n, void *stream);
 /* Launch-shape knobs for sweeps and for the tests that show the results do not depend on them; value 0 restores
  * the built-in choice.  Keys: "norm_quant_nchunk" (1/2/4/8 16-byte chunks per lane), "norm_quant_threads" (lanes
  * per row), "norm_quant_rows" (1 or 2 rows per workgroup), "norm_quant_paired_stores" (0/1), "norm_quant_lds_pad"
- * (bytes of idle LDS per workgroup), "rope_block_threads" (64/128/256/512).  Unknown keys or values return
+ * (bytes of idle LDS per workgroup), "norm_quant_row_group_shift" (log2 of the run of consecutive rows one XCD takes;
+ * -1, not 0, restores the built-in rule), "rope_block_threads" (64/128/256/512).  Unknown keys or values return
  * GPUK_ERR_INVALID_ARG.  Not part of the reference. */
 int gpuk_set_tuning(const char *key, int value);
 

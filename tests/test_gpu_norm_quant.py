@@ -179,6 +179,23 @@ def test_launch_shape_variants(device, threads, nchunk, paired, rows):
         capi.set_tuning("norm_quant_rows", 0)
 
 
+@pytest.mark.parametrize("shift", [-1, 0, 1, 3, 6, 7])
+def test_row_runs_per_xcd(device, shift):
+    """Which workgroup takes which row (runs of 2^shift consecutive rows per XCD, identity past the last full
+    round) is a tuning choice only.  -1 is the built-in rule, which groups at these row sizes from 1024 rows on."""
+    from gpuk_amd import capi
+
+    print(f"case row runs shift={shift}", flush=True)
+    capi.set_tuning("norm_quant_row_group_shift", shift)
+    try:
+        for tokens, hidden in ((1100, 4096), (1027, 8192), (301, 1032), (2048, 8192)):
+            inp = workloads.norm_quant_inputs(tokens, hidden, seed=shift + hidden, res_sigma=2.0, outlier_frac=0.01)
+            for quant in (0, 1):
+                check(inp, quant, run_capi(inp, quant, device), tag=f"[runs 2^{shift} {tokens}x{hidden} q{quant}]")
+    finally:
+        capi.set_tuning("norm_quant_row_group_shift", -1)
+
+
 def test_config1_static_per_tensor(device):
     """tokens=128, hidden=4096, static scale = amax(normed)/448 computed once by the oracle."""
     inp = workloads.config1()
