@@ -246,6 +246,42 @@ def main():
                             "frac_of_8TBps": round(nbytes / (burst * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                             "algorithmic_bytes": nbytes}
 
+        # the two-stream op at the reference script's shape (test/test_fused_rope_rms_2way.py:223-246), and the no-KV
+        # mRoPE op on the Qwen2-VL-like shape
+        B2, T0, T1, Hq2, Hk2, D2 = 2, 678, 3608, 24, 25, 128
+        g2 = torch.Generator(device=dev).manual_seed(7)
+        mk = lambda *shape: torch.randn(shape, device=dev, generator=g2).to(torch.bfloat16)
+        ins2 = [(mk(B2, T0, Hq2, D2), mk(B2, T0, Hk2, D2), mk(B2, T1, Hq2, D2), mk(B2, T1, Hk2, D2)) for _ in range(3)]
+        w2 = [mk(D2) for _ in range(4)]
+        cs0, cs1 = mk(T0, D2), mk(T1, D2)
+        out2 = (torch.empty((B2, T0 + T1, Hq2, D2), dtype=torch.bfloat16, device=dev),
+                torch.empty((B2, T0 + T1, Hk2, D2), dtype=torch.bfloat16, device=dev))
+
+        def two_way_call(i=0):
+            q0, k0_, q1, k1_ = ins2[i % 3]
+            capi.rope_rms_2way(q0, k0_, q1, k1_, *w2, cs0, cs1, B2, T0, T1, Hq2, Hk2, D2, False, 1e-6, *out2)
+
+        nb2 = 2 * (B2 * (T0 + T1) * (Hq2 + Hk2) * D2 * 2) + (T0 + T1) * D2 * 2 + 4 * D2 * 2
+        ms2 = event_time_ms(two_way_call, 100)
+        extras["rope_2way_B2_678+3608"] = {"us_per_call": round(ms2 * 1e3, 2), "GBps": round(nb2 / (ms2 * 1e-3) / 1e9, 1),
+                                           "frac_of_8TBps": round(nb2 / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                           "algorithmic_bytes": nb2}
+        r4 = workloads.config4()
+        qw4, kw4, cs4, pos4 = (t.to(dev) for t in (r4.qw, r4.kw, r4.cos_sin, r4.positions))
+        qkv4 = [r4.qkv.to(dev).clone() for _ in range(4)]
+
+        def mrope_inplace_call(i=0):
+            capi.rope_rms(qkv4[i % 4], qw4, kw4, cs4, pos4, r4.num_tokens, r4.num_heads_q, r4.num_heads_k, r4.num_heads_v,
+                          r4.head_size, r4.is_neox, r4.eps, r4.mrope_section, r4.is_interleaved)
+
+        nb4 = workloads.rope_inplace_bytes(r4.num_tokens, r4.num_heads_q, r4.num_heads_k, r4.head_size, 3)
+        ms4 = event_time_ms(mrope_inplace_call, 100)
+        extras["mrope_inplace_qwen2vl_T8192"] = {"us_per_call": round(ms4 * 1e3, 2),
+                                                 "GBps": round(nb4 / (ms4 * 1e-3) / 1e9, 1),
+                                                 "frac_of_8TBps": round(nb4 / (ms4 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                                 "algorithmic_bytes": nb4}
+        del ins2, out2, qkv4
+
         # decode shapes: per call, eager (host launch overhead included) and replayed from a HIP graph of 20 calls on
         # 20 distinct buffer sets (GPU-side cost)
         decode = {}
