@@ -176,8 +176,15 @@ struct RopeUnit {
         st.head = min(head_raw, heads_qk - 1);
         st.is_q = st.head < a.hq;
         const uint16_t *src = st.token_in + (int64_t)st.head * D;
-        st.xa = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c0(sub)));
-        st.xb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c1(sub)));
+        // streamed when the results go elsewhere; in place the same lines are written a moment later, and keeping
+        // them in L2 measured 2 % faster
+        if constexpr (SETKV) {
+            st.xa = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c0(sub)));
+            st.xb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c1(sub)));
+        } else {
+            st.xa = *reinterpret_cast<const u32x4 *>(src + c0(sub));
+            st.xb = *reinterpret_cast<const u32x4 *>(src + c1(sub));
+        }
 
         // this wave's share of the token's V row: chunk u*64 + lane (and further strides of units_per_token*64)
         if constexpr (SETKV) {
