@@ -432,7 +432,6 @@ __global__ void __launch_bounds__(256) rope_rms_2way_kernel(const TwoWayArgs a) 
     const uint32_t unit_in_seg = unit - (seg ? a.unit_end[seg - 1] : 0u);
     const int kind = seg & 1, stream_id = seg >> 1;  // q|k, stream 0|1
     const uint32_t heads = a.heads[kind], rows = a.rows[seg];
-    const int tokens_seg = stream_id ? a.tokens1 : a.tokens0;
     const int batch = blockIdx.y;
 
     const int lane = threadIdx.x & 63, sub = lane % LPH, hl = lane / LPH;
@@ -462,7 +461,60 @@ __global__ void __launch_bounds__(256) rope_rms_2way_kernel(const TwoWayArgs a) 
         *reinterpret_cast<u32x4 *>(dst + c0) = oa;
         *reinterpret_cast<u32x4 *>(dst + c1) = ob;
     }
-    (void)tokens_seg;
+}
+
+// fp32 form of the two-stream op (the reference dispatches float here too: src/ops/fused_rope.cpp:197-200): one wave
+// per (token, head) row of a segment, lane l owns rotation pairs l, l+64, ...; plain fp32 arithmetic, every product
+// rounded before the add.  The host counts one unit per row for this kernel.
+template <int D, bool NEOX>
+__global__ void __launch_bounds__(256) rope_rms_2way_f32_kernel(const TwoWayArgs a) {
+    constexpr int HALF = D / 2;
+    constexpr int PPL = (HALF + 63) / 64;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t unit = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (unit >= a.unit_end[3]) return;
+    const int seg = (unit >= a.unit_end[0]) + (unit >= a.unit_end[1]) + (unit >= a.unit_end[2]);
+    const uint32_t row = unit - (seg ? a.unit_end[seg - 1] : 0u);
+    const int kind = seg & 1, stream_id = seg >> 1;
+    const uint32_t heads = a.heads[kind], rows = a.rows[seg];
+    const int batch = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const uint32_t token = a.heads_magic[kind] ? __umulhi(row, a.heads_magic[kind]) : row;
+    const uint32_t head = row - token * heads;
+
+    const float *src = static_cast<const float *>(a.in[seg]) + ((int64_t)batch * rows + row) * D;
+    const float *w = static_cast<const float *>(a.w[seg]);
+    const float *table = static_cast<const float *>(a.cos_sin[stream_id]) + (int64_t)token * D;
+    const int64_t out_token = (int64_t)batch * (a.tokens0 + a.tokens1) + (stream_id ? a.tokens0 : 0) + token;
+    float *dst = static_cast<float *>(a.out[kind]) + (out_token * heads + head) * D;
+
+    float x1[PPL], x2[PPL];
+    int i1[PPL], i2[PPL];
+    bool live[PPL];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < PPL; ++k) {
+        const int p = lane + 64 * k;
+        live[k] = p < HALF;
+        const int pc = live[k] ? p : 0;
+        i1[k] = NEOX ? pc : 2 * pc;
+        i2[k] = NEOX ? pc + HALF : 2 * pc + 1;
+        x1[k] = live[k] ? src[i1[k]] : 0.f;
+        x2[k] = live[k] ? src[i2[k]] : 0.f;
+        ss = __builtin_fmaf(x1[k], x1[k], ss);
+        ss = __builtin_fmaf(x2[k], x2[k], ss);
+    }
+    ss = wave_allreduce<SumOp>(ss);
+    const float rstd = 1.0f / sqrtf(ss * (1.0f / D) + a.eps);
+#pragma unroll
+    for (int k = 0; k < PPL; ++k) {
+        if (!live[k]) continue;
+        const int f = lane + 64 * k;
+        const float c = table[f], s = table[HALF + f];
+        const float n1 = w[i1[k]] * (x1[k] * rstd), n2 = w[i2[k]] * (x2[k] * rstd);
+        dst[i1[k]] = n1 * c - n2 * s;
+        dst[i2[k]] = n2 * c + n1 * s;
+    }
 }
 
 template <typename T, int D>
@@ -471,6 +523,23 @@ int launch_2way(const TwoWayArgs &a, bool neox, unsigned batch, hipStream_t stre
     if (neox) rope_rms_2way_kernel<T, D, true><<<grid, 256, 0, stream>>>(a);
     else rope_rms_2way_kernel<T, D, false><<<grid, 256, 0, stream>>>(a);
     return hip_status(hipGetLastError());
+}
+
+template <int D>
+int launch_2way_f32(const TwoWayArgs &a, bool neox, unsigned batch, hipStream_t stream) {
+    const dim3 grid((a.unit_end[3] + 3) / 4, batch);
+    if (neox) rope_rms_2way_f32_kernel<D, true><<<grid, 256, 0, stream>>>(a);
+    else rope_rms_2way_f32_kernel<D, false><<<grid, 256, 0, stream>>>(a);
+    return hip_status(hipGetLastError());
+}
+
+int launch_2way_f32_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned batch, hipStream_t stream) {
+    switch (D) {
+        case 64: return launch_2way_f32<64>(a, neox, batch, stream);
+        case 128: return launch_2way_f32<128>(a, neox, batch, stream);
+        case 256: return launch_2way_f32<256>(a, neox, batch, stream);
+        default: return GPUK_ERR_UNSUPPORTED;
+    }
 }
 
 template <typename T>
@@ -672,9 +741,9 @@ extern "C" int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1
     using namespace gpuk;
     if (batch_size < 0 || num_tokens0 < 0 || num_tokens1 < 0 || num_heads_q < 0 || num_heads_k < 0) return GPUK_ERR_INVALID_ARG;
     if (head_size != 64 && head_size != 128 && head_size != 256) return GPUK_ERR_UNSUPPORTED;
-    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16) return GPUK_ERR_UNSUPPORTED;
+    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32) return GPUK_ERR_UNSUPPORTED;
     if (batch_size > 65535) return GPUK_ERR_UNSUPPORTED;  // grid.y
-    const int64_t hpw = 64 / (head_size / 16);
+    const int64_t hpw = dtype == GPUK_DTYPE_F32 ? 1 : 64 / (head_size / 16);  // rows (heads) per wave
     const int64_t rows[4] = {num_tokens0 * num_heads_q, num_tokens0 * num_heads_k, num_tokens1 * num_heads_q,
                              num_tokens1 * num_heads_k};
     const void *ins[4] = {q0, k0, q1, k1};
@@ -712,6 +781,7 @@ extern "C" int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1
     a.eps = eps;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool neox = !is_interleaved;  // reference: fused_rope.cpp:168-227 dispatches the NeoX kernel when !is_interleaved
+    if (dtype == GPUK_DTYPE_F32) return launch_2way_f32_head_size(a, head_size, neox, (unsigned)batch_size, s);
     if (dtype == GPUK_DTYPE_BF16) return launch_2way_head_size<BF16>(a, head_size, neox, (unsigned)batch_size, s);
     return launch_2way_head_size<FP16>(a, head_size, neox, (unsigned)batch_size, s);
 }

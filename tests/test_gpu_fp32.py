@@ -135,3 +135,24 @@ def test_rope_set_kv_fp32(device, kv_dtype, mrope):
     assert_bits_equal(raw(kc[untouched]), raw(k0[untouched]), "untouched k slots")
     assert_bits_equal(raw(vc[untouched]), raw(v0[untouched]), "untouched v slots")
     assert torch.equal(qkv.cpu(), inp.qkv), "set_kv must not modify qkv"
+
+
+@pytest.mark.parametrize("head_size", [64, 128, 256])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_rope_2way_fp32(device, head_size, interleaved):
+    import gpuk_amd as gpuk
+
+    print(f"case fp32 2way D={head_size} il={interleaved}", flush=True)
+    B, T0, T1, Hq, Hk = 2, 19, 45, 3, 5
+    g = torch.Generator().manual_seed(head_size + interleaved)
+    mk = lambda *shape: torch.randn(shape, generator=g, dtype=torch.float32)
+    q0, k0, q1, k1 = mk(B, T0, Hq, head_size), mk(B, T0, Hk, head_size), mk(B, T1, Hq, head_size), mk(B, T1, Hk, head_size)
+    ws = [1 + 0.2 * mk(head_size) for _ in range(4)]
+    cs0, cs1 = mk(T0, head_size), mk(T1, head_size)
+    dev = lambda t: t.to(device)
+    out_q, out_k = gpuk.fused_rope_rms_2way(dev(q0), dev(k0), dev(q1), dev(k1), *(dev(w) for w in ws), dev(cs0), dev(cs1),
+                                            B, T0, T1, Hq, Hk, head_size, interleaved, 1e-6)
+    torch.cuda.synchronize()
+    ref_q, ref_k = O.rope_rms_2way_ref(q0, k0, q1, k1, *ws, cs0, cs1, B, T0, T1, Hq, Hk, head_size, interleaved, 1e-6)
+    close32(out_q, ref_q, "out_q01")
+    close32(out_k, ref_k, "out_k01")
