@@ -388,10 +388,10 @@ int g_row_group_shift = -1;  // -1 = heuristic, else log2 of the run of consecut
 int g_lds_pad = 0;        // unused dynamic LDS bytes per workgroup: caps the workgroups resident per CU
 int g_paired = 0;         // 16-byte paired code stores (measured no faster than 8-byte stores; kept selectable)
 
-// Lanes per row and chunks per lane.  Measured on MI355X with the traffic pattern alone: 512-lane
-// workgroups with 2 chunks per lane stream best for rows of 4096..8192 elements; shorter rows use one
-// chunk per lane; few rows (decode) spread each row over as many lanes as possible to shorten the
-// dependent load -> reduce -> reduce -> store chain.
+// Lanes per row and chunks per lane.  Measured on MI355X over rows of 1024 .. 16384 elements: two chunks per lane
+// on as many lanes as that needs (up to 1024) streams best or ties everywhere (1-6 % over one or four chunks per
+// lane), unless rounding up to whole waves would idle more lanes that way; longer rows double the chunks per lane; few rows (decode) spread each row over as many lanes as possible
+// to shorten the dependent load -> reduce -> reduce -> store chain.
 void pick_shape(int64_t tokens, int chunks_per_row, int *threads, int *nchunk) {
     auto fits = [&](int n) { return (int64_t)n * kMaxThreads >= chunks_per_row; };
     int n;
@@ -400,8 +400,10 @@ void pick_shape(int64_t tokens, int chunks_per_row, int *threads, int *nchunk) {
     } else if (tokens <= 256) {
         n = 1;
     } else {
-        n = 1;
-        while (n < 8 && chunks_per_row > 512 * n) n *= 2;
+        // one chunk per lane only where two would leave more lanes idle after rounding up to whole waves
+        const int lanes1 = round_up(chunks_per_row, 64), lanes2 = round_up((chunks_per_row + 1) / 2, 64);
+        n = (2 * lanes2 > lanes1 && lanes1 <= kMaxThreads) ? 1 : 2;
+        while (n < 8 && chunks_per_row > kMaxThreads * n) n *= 2;
     }
     while (n < 8 && !fits(n)) n *= 2;
     if (!fits(n)) {
@@ -437,10 +439,10 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
     const dim3 grid2((unsigned)((tokens + rows - 1) / rows));
     const float rcp_hidden = 1.0f / hf;
     const int tok = (int)tokens;
-    // Runs of 64 rows per XCD: measured +1.1 % at 16 KiB rows and +1 % at 8 KiB rows (8192 rows), neutral for fewer
-    // rows, and 1-10 % slower for rows of any other size (2 KiB, 4 KiB, 10 KiB, 14 KiB, 32 KiB), hence the narrow rule.
+    // Runs of 64 rows per XCD: measured +1.1 % for 16 KiB rows (8192 rows); neutral or 1-10 % slower for every other
+    // row size tried (2, 3, 4, 8, 10, 14, 32 KiB) and for fewer rows, hence the narrow rule.
     const int64_t row_bytes = hidden * 2;
-    int group_shift = (row_bytes == 8192 || row_bytes == 16384) && grid2.x >= 1024 ? 6 : 0;
+    int group_shift = row_bytes == 16384 && grid2.x >= 1024 ? 6 : 0;
     if (g_row_group_shift >= 0) group_shift = g_row_group_shift;
     const int remap_end = group_shift > 0 ? (int)((grid2.x >> (3 + group_shift)) << (3 + group_shift)) : 0;
 #define GPUK_LAUNCH_NQ(N, PAIRED, ROWS)                                                                       \

@@ -182,7 +182,7 @@ def test_launch_shape_variants(device, threads, nchunk, paired, rows):
 @pytest.mark.parametrize("shift", [-1, 0, 1, 3, 6, 7])
 def test_row_runs_per_xcd(device, shift):
     """Which workgroup takes which row (runs of 2^shift consecutive rows per XCD, identity past the last full
-    round) is a tuning choice only.  -1 is the built-in rule, which groups at these row sizes from 1024 rows on."""
+    round) is a tuning choice only.  -1 is the built-in rule, which groups 16 KiB rows from 1024 rows on."""
     from gpuk_amd import capi
 
     print(f"case row runs shift={shift}", flush=True)
