@@ -202,8 +202,8 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
                         q[j] = div_by_rcp(v[j], scale, rcp);
-                        if constexpr (kClamp) q[j] = clamp_sym(q[j], fp8_max);
                     }
+                    if constexpr (kClamp) clamp8_sym(q, fp8_max);
                     return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
                 };
                 if constexpr (PAIRED) {

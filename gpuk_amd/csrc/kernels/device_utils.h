@@ -170,6 +170,21 @@ __device__ __forceinline__ float clamp_sym(float v, float bound) {
     return v != v ? v : c;
 }
 
+// clamp_sym over 8 values, done only if one of them is out of range (rare): the test costs four v_max3_f32, the
+// clamps 24 instructions.  A NaN does not trigger the clamp (fmax drops it) and needs none: the fp8 converter maps
+// NaN to NaN.
+__device__ __forceinline__ void clamp8_sym(float (&q)[8], float bound) {
+    const float m01 = __builtin_fmaxf(__builtin_fabsf(q[0]), __builtin_fabsf(q[1]));
+    const float m23 = __builtin_fmaxf(__builtin_fabsf(q[2]), __builtin_fabsf(q[3]));
+    const float m45 = __builtin_fmaxf(__builtin_fabsf(q[4]), __builtin_fabsf(q[5]));
+    const float m67 = __builtin_fmaxf(__builtin_fabsf(q[6]), __builtin_fabsf(q[7]));
+    const float m = __builtin_fmaxf(__builtin_fmaxf(m01, m23), __builtin_fmaxf(m45, m67));
+    if (__builtin_expect(m > bound, 0)) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q[j] = clamp_sym(q[j], bound);
+    }
+}
+
 // Correctly rounded fp32 quotient a/b given rcp = RN(1/b): one multiply and two fused
 // multiply-adds (Markstein's correction step).  Valid while a/b, the residual and rcp stay in the
 // normal range and b > 0; callers guard the range of b once per row and fall back to `/` outside it.

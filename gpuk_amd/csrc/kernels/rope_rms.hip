@@ -77,9 +77,10 @@ __device__ __forceinline__ u32x2 quantize_chunk(const u32x4 &v, float scale, flo
         const float a = FAST ? div_by_rcp(P::lo(v[j]), scale, rcp) : P::lo(v[j]) / scale;
         const float b = FAST ? div_by_rcp(P::hi(v[j]), scale, rcp) : P::hi(v[j]) / scale;
         const uint32_t w = P::pack(a, b);
-        q[2 * j] = clamp_sym(P::lo(w), kE4M3Max);
-        q[2 * j + 1] = clamp_sym(P::hi(w), kE4M3Max);
+        q[2 * j] = P::lo(w);
+        q[2 * j + 1] = P::hi(w);
     }
+    clamp8_sym(q, kE4M3Max);
     return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
 }
 __device__ __forceinline__ bool scale_is_fast(float s) { return s >= 0x1p-60f && s <= 0x1p60f; }

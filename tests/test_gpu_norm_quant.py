@@ -335,3 +335,16 @@ def test_increment_floats_calibration_kernel(device):
         want = torch.arange(n + 4, dtype=torch.float32)
         want[:n] += 1
         assert torch.equal(data.cpu(), want), n
+
+
+@pytest.mark.parametrize("fp8_max", [448.0, 240.0])
+def test_static_scale_too_small_saturates(device, fp8_max):
+    """A static scale 8 times too small: most quotients exceed fp8_max and are clipped to it, as the oracle's clamp
+    does (gpuk/__init__.py:160-162), instead of overflowing to NaN in the conversion."""
+    inp = workloads.norm_quant_inputs(64, 4096, seed=17, res_sigma=1.5)
+    static = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) / 64.0
+    got = run_capi(inp, 3, device, fp8_max=fp8_max, static_scale=static)
+    check(inp, 3, got, fp8_max=fp8_max, static_scale=static, tag=f"[saturating static scale, max {fp8_max}]")
+    codes = got[1].cpu().view(torch.uint8) & 0x7F
+    top = 0x7E if fp8_max == 448.0 else 0x77
+    assert (codes == top).float().mean() > 0.3 and (codes <= top).all()

@@ -298,3 +298,21 @@ def test_op_rejects_bad_arguments(device):
                                 [16, 16, 16], False, 1e-6)
     with pytest.raises(RuntimeError):   # unsupported head size (reference: assert rope_rms_impl.h:473)
         gpuk.fused_rope_rms(qkv, qw, kw, cs, pos, 8, 4, 4, 4, 96, True, 1e-6)
+
+
+def test_fp8_cache_saturates_out_of_range_values(device):
+    """With scales far too small most quotients exceed 448.  The kernel clips them to +-448, as the reference kernel
+    clips at its maximum (src/impl/rope_rms_impl.h:109-118 -> float8.h), where torch's cast would give NaN above 464:
+    expected codes = e4m3fn(clamp(rT(o / scale), +-448)) from the oracle's rotated K and raw V."""
+    print("case fp8 cache saturation", flush=True)
+    inp = make(40, 8, 128, True, seed=91, fp8=True, hk=4, hv=4)
+    inp.k_scale, inp.v_scale = 1.0 / 512.0, 1.0 / 300.0
+    q_out, kc, vc, (k0, v0) = run_set_kv(inp, device)
+    q, k, v = O.rope_rms_ref(inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, 40, 8, 4, 4, 128, True, inp.eps)
+    want_k = (k / inp.k_scale).clamp(-448, 448).to(torch.float8_e4m3fn)
+    want_v = (v / inp.v_scale).clamp(-448, 448).to(torch.float8_e4m3fn)
+    got_k, got_v = kc.cpu()[inp.kv_loc], vc.cpu()[inp.kv_loc]
+    assert ((want_k.view(torch.uint8) & 0x7F) == 0x7E).float().mean() > 0.3      # the test does saturate
+    assert not ((got_k.view(torch.uint8) & 0x7F) == 0x7F).any() and not ((got_v.view(torch.uint8) & 0x7F) == 0x7F).any()
+    assert_codes_close(got_k, want_k, "saturated k codes")
+    assert_bits_equal(got_v.view(torch.uint8), want_v.view(torch.uint8), "saturated v codes")
