@@ -67,6 +67,32 @@ __device__ __forceinline__ float elem(const u32x4 &v, int e) {  // element e (0.
     return (e & 1) ? Pack16<T>::hi(v[e >> 1]) : Pack16<T>::lo(v[e >> 1]);
 }
 
+// A lane's two chunks sit at elements 8*sub and D/2 + 8*sub of its head in both styles, so that every load and store
+// instruction of a wave covers whole 128-byte lines.  NeoX: the chunks hold x1 and x2 of rotary frequencies
+// 8*sub .. 8*sub+7.  GPT-J: each dword is an (x1, x2) pair; the first chunk holds frequencies 4*sub .. 4*sub+3, the
+// second D/4 + 4*sub .. D/4 + 4*sub+3.  The cos (or sin) values of the lane's 8 frequencies, first chunk's first:
+template <int D, bool NEOX>
+__device__ __forceinline__ u32x4 load_trig(const uint16_t *row, int sub) {  // row = cos (or sin) half of a table row
+    if constexpr (NEOX) {
+        return *reinterpret_cast<const u32x4 *>(row + 8 * sub);
+    } else {
+        const u32x2 lo = *reinterpret_cast<const u32x2 *>(row + 4 * sub);
+        const u32x2 hi = *reinterpret_cast<const u32x2 *>(row + D / 4 + 4 * sub);
+        return u32x4{lo[0], lo[1], hi[0], hi[1]};
+    }
+}
+// ... and the matching 8 bits of a frequency bitmap (bit f = frequency f)
+template <int D, bool NEOX>
+__device__ __forceinline__ uint32_t trig_bits(const uint32_t (&bitmap)[4], int sub) {
+    if constexpr (NEOX) {
+        const int f = 8 * sub;
+        return (bitmap[f >> 5] >> (f & 31)) & 0xffu;
+    } else {
+        const int f0 = 4 * sub, f1 = D / 4 + 4 * sub;
+        return ((bitmap[f0 >> 5] >> (f0 & 31)) & 0xfu) | (((bitmap[f1 >> 5] >> (f1 & 31)) & 0xfu) << 4);
+    }
+}
+
 // 8 codes = e4m3fn(clamp(rT(v / scale))) for one chunk; `rcp` is RN(1/scale) and is used when FAST
 template <typename T, bool FAST>
 __device__ __forceinline__ u32x2 quantize_chunk(const u32x4 &v, float scale, float rcp) {
@@ -87,7 +113,7 @@ __device__ __forceinline__ bool scale_is_fast(float s) { return s >= 0x1p-60f &&
 
 // RMSNorm of one head (D/16 lanes x two chunks) followed by the rotation, for the lane's two chunks.
 //   NeoX : chunk a holds x1 for the lane's 8 frequencies, chunk b the matching x2.
-//   GPT-J: each dword is one (x1, x2) pair; chunk a uses the lane's frequencies 0-3, chunk b 4-7.
+//   GPT-J: each dword is one (x1, x2) pair; chunk a uses cos/sin values 0-3 of the lane, chunk b values 4-7.
 template <typename T, int D, bool NEOX>
 __device__ __forceinline__ void norm_rotate(const u32x4 &xa, const u32x4 &xb, const u32x4 &wa, const u32x4 &wb,
                                             const u32x4 &cosv, const u32x4 &sinv, float eps, u32x4 &oa, u32x4 &ob) {
@@ -156,10 +182,9 @@ struct RopeUnit {
     static constexpr int HPW = 64 / LPH;  // heads per wave
     static constexpr int HALF = D / 2;
 
-    // element offsets of a lane's two chunks inside a head (NeoX: x1 chunk and the chunk D/2 further; GPT-J: two
-    // adjacent chunks) and of its cos / sin chunks inside a table row
-    static __device__ __forceinline__ int c0(int sub) { return NEOX ? 8 * sub : 16 * sub; }
-    static __device__ __forceinline__ int c1(int sub) { return NEOX ? HALF + 8 * sub : 16 * sub + 8; }
+    // element offsets of a lane's two chunks inside a head
+    static __device__ __forceinline__ int c0(int sub) { return 8 * sub; }
+    static __device__ __forceinline__ int c1(int sub) { return HALF + 8 * sub; }
 
     // Issues every load of the unit; nothing is waited for.
     static __device__ __forceinline__ void issue_loads(const RopeArgs &a, uint32_t unit, int lane, UnitState &st) {
@@ -210,21 +235,19 @@ struct RopeUnit {
     static __device__ __forceinline__ void issue_table_loads(const RopeArgs &a, int lane, UnitState &st) {
         if (!st.live) return;
         const int sub = lane % LPH;
-        const int fc = 8 * sub;
         const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin);
         const int64_t p0 = st.p0;
-        st.cosv = *reinterpret_cast<const u32x4 *>(table + p0 * D + fc);
-        st.sinv = *reinterpret_cast<const u32x4 *>(table + p0 * D + HALF + fc);
+        st.cosv = load_trig<D, NEOX>(table + p0 * D, sub);
+        st.sinv = load_trig<D, NEOX>(table + p0 * D + HALF, sub);
         if constexpr (AXES == 3) {
             const int64_t p1 = st.p1, p2 = st.p2;
             if (p1 != p0 || p2 != p0) {  // wave-uniform; text tokens carry three equal positions
-                const u32x4 cos1 = *reinterpret_cast<const u32x4 *>(table + p1 * D + fc);
-                const u32x4 sin1 = *reinterpret_cast<const u32x4 *>(table + p1 * D + HALF + fc);
-                const u32x4 cos2 = *reinterpret_cast<const u32x4 *>(table + p2 * D + fc);
-                const u32x4 sin2 = *reinterpret_cast<const u32x4 *>(table + p2 * D + HALF + fc);
-                // 8 axis bits for frequencies fc .. fc+7 (fc is a multiple of 8, so they share a word)
-                const uint32_t b1 = (a.axis1[fc >> 5] >> (fc & 31)) & 0xffu;
-                const uint32_t b2 = (a.axis2[fc >> 5] >> (fc & 31)) & 0xffu;
+                const u32x4 cos1 = load_trig<D, NEOX>(table + p1 * D, sub);
+                const u32x4 sin1 = load_trig<D, NEOX>(table + p1 * D + HALF, sub);
+                const u32x4 cos2 = load_trig<D, NEOX>(table + p2 * D, sub);
+                const u32x4 sin2 = load_trig<D, NEOX>(table + p2 * D + HALF, sub);
+                // the axis bits of the lane's 8 frequencies, in the order of the loaded values
+                const uint32_t b1 = trig_bits<D, NEOX>(a.axis1, sub), b2 = trig_bits<D, NEOX>(a.axis2, sub);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t m1 = halves_mask(b1 >> (2 * j)), m2 = halves_mask(b2 >> (2 * j));
@@ -442,7 +465,7 @@ __global__ void __launch_bounds__(256) rope_rms_2way_kernel(const TwoWayArgs a) 
     const uint32_t token = a.heads_magic[kind] ? __umulhi(row, a.heads_magic[kind]) : row;
     const uint32_t head = row - token * heads;
 
-    const int c0 = NEOX ? 8 * sub : 16 * sub, c1 = NEOX ? HALF + 8 * sub : 16 * sub + 8, fc = 8 * sub;
+    const int c0 = 8 * sub, c1 = HALF + 8 * sub;
     const uint16_t *src = static_cast<const uint16_t *>(a.in[seg]) + ((int64_t)batch * rows + row) * D;
     const u32x4 xa = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c0));
     const u32x4 xb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c1));
@@ -450,8 +473,8 @@ __global__ void __launch_bounds__(256) rope_rms_2way_kernel(const TwoWayArgs a) 
     const u32x4 wa = *reinterpret_cast<const u32x4 *>(wsrc + c0);
     const u32x4 wb = *reinterpret_cast<const u32x4 *>(wsrc + c1);
     const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin[stream_id]) + (int64_t)token * D;
-    const u32x4 cosv = *reinterpret_cast<const u32x4 *>(table + fc);
-    const u32x4 sinv = *reinterpret_cast<const u32x4 *>(table + HALF + fc);
+    const u32x4 cosv = load_trig<D, NEOX>(table, sub);
+    const u32x4 sinv = load_trig<D, NEOX>(table + HALF, sub);
     __builtin_amdgcn_sched_barrier(0);
 
     u32x4 oa, ob;
