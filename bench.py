@@ -9,7 +9,8 @@ cache can serve a repeat.  Prints ONE JSON line:
 
   value      achieved HBM GB/s over the K timed steps = algorithmic bytes (7*T*H + 4*T + 2*H) / wall time
   roofline   the same kernel timed per launch with HIP events on the launch stream, against 8 TB/s
-  cpu_baseline  the restated torch reference on the host's cores, on a bounded row sample of the same batch
+  cpu_baseline  the restated torch reference on the host's cores, on a bounded row sample of the same batch; where
+             oracle/_ref was built, also the reference's own kernels timed on this GPU beside this repository's
   extras     secondary figures: copy-kernel ceiling, the RoPE + KV-write kernel on its two configurations,
              decode-shape latencies (us/call)
 """
@@ -204,6 +205,48 @@ def main():
                         "sample": f"restated torch reference (oracle/torch_oracle.py) on CPU tensors, first {rows} of {T} "
                                   f"rows x {H}, median of {len(times)} calls over {time.perf_counter() - t_start:.1f} s "
                                   f"({t_med * 1e3:.0f} ms/call); host reports {ncores} cpus"}
+
+        # Second baseline, same leg: the reference repository's own kernels (oracle/_ref, built from the reference's
+        # headers where a checkout exists) timed on this GPU on the same inputs and buffer rotation.  For the norm-quant
+        # path that is the reference's epilogue device code under a one-GPU caller (its kernels need 2+ GPUs), with the
+        # reference's fp8 maximum of 240; for the rope path it is the reference's kernel as the reference launches it.
+        from oracle import ref_kernels
+
+        if ref_kernels.available():
+            ref = {}
+
+            def ref_norm_quant_us(tokens, hidden):
+                d = workloads.config2(tokens, hidden)
+                g_ = d.gamma.to(dev)
+                bufs = [(d.x.to(dev), d.residual.to(dev), torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev),
+                         torch.empty((tokens, hidden), dtype=torch.float8_e4m3fn, device=dev),
+                         torch.empty((tokens, 1), dtype=torch.float32, device=dev)) for _ in range(3)]
+                theirs = event_time_ms(lambda i=0: ref_kernels.epilogue_rows(*bufs[i % 3][:2], g_, *bufs[i % 3][2:], eps, 1), 50)
+                ours = event_time_ms(lambda i=0: capi.add_rmsnorm_quant(*bufs[i % 3][:2], g_, *bufs[i % 3][2:], eps, 1, 240.0), 50)
+                return round(theirs * 1e3, 2), round(ours * 1e3, 2)
+
+            for tokens, hidden in ((8192, 8192), (8192, 4096)):
+                theirs, ours = ref_norm_quant_us(tokens, hidden)
+                ref[f"add_rmsnorm_quant_{tokens}x{hidden}_us"] = {"reference_epilogue": theirs, "this_repository": ours}
+
+            def ref_rope_us(r):
+                k0, v0 = r.new_cache()
+                qw, kw, cs, pos, loc = (t.to(dev) for t in (r.qw, r.kw, r.cos_sin, r.positions, r.kv_loc))
+                bufs = [(r.qkv.to(dev).clone(), torch.empty((r.num_tokens, r.num_heads_q, r.head_size), dtype=torch.bfloat16,
+                                                            device=dev), k0.to(dev), v0.to(dev)) for _ in range(4)]
+                shape = (r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size, r.is_neox, r.eps)
+                theirs = event_time_ms(lambda i=0: ref_kernels.mrope_rms_set_kv(
+                    bufs[i % 4][0], qw, kw, cs, pos, *shape, *bufs[i % 4][1:], loc, r.k_scale, r.v_scale, r.mrope_section,
+                    r.is_interleaved), 50)
+                ours = event_time_ms(lambda i=0: capi.rope_rms_set_kv(
+                    bufs[i % 4][0], qw, kw, cs, pos, *shape, *bufs[i % 4][1:], loc, r.k_scale, r.v_scale, r.mrope_section,
+                    r.is_interleaved), 50)
+                return round(theirs * 1e3, 2), round(ours * 1e3, 2)
+
+            for name, r in (("rope_kv_qwen3_T4096_us", workloads.config3()), ("mrope_kv_qwen2vl_T8192_us", workloads.config4())):
+                theirs, ours = ref_rope_us(r)
+                ref[name] = {"reference_kernel": theirs, "this_repository": ours}
+            cpu_baseline["reference_kernels_on_this_gpu"] = ref
 
     # ------------------------------------------------------------------ secondary figures
     extras = {}

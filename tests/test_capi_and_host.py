@@ -229,3 +229,20 @@ def test_mut_overloads_have_meta_kernels():
     qkv = torch.empty((4, 6, 64), dtype=torch.bfloat16, device="meta")
     pos = torch.empty((4,), dtype=torch.int64, device="meta")
     assert gpuk_amd.traceable.fused_rope_rms(qkv, g, g, x, pos, 4, 2, 2, 2, 64, True, 1e-6) is None
+
+
+def test_reference_kernel_library_exports_its_entry_points():
+    """oracle/_ref/libgpuk_ref.so (the reference's own kernels, compiled where a reference checkout exists) loads and
+    exports the four entry points the GPU tests call.  Skipped where it was never built."""
+    from oracle import ref_kernels
+
+    if not ref_kernels.available():
+        pytest.skip("oracle/_ref/libgpuk_ref.so not built")
+    import torch  # noqa: F401  (its HIP runtime first, as for the product library)
+
+    L = ref_kernels.lib()
+    for name in ("gpuk_ref_rope_rms", "gpuk_ref_mrope_rms_set_kv", "gpuk_ref_rope_rms_2way", "gpuk_ref_epilogue_rows"):
+        assert hasattr(L, name), name
+    # argument refusal happens before any launch
+    assert L.gpuk_ref_epilogue_rows(None, None, None, None, None, None, 0, 4096, 1e-6, 1, None) == -1
+    assert L.gpuk_ref_rope_rms(None, None, None, None, None, 0, 1, 1, 4, 2, 2, 2, 96, 1, None, 0, 1e-6, None) == -1
