@@ -26,8 +26,10 @@ exhaustive torch-CPU table over all 65536 bf16 patterns; RMSNorm against an fp64
 brute force and scale invariances; the double bf16 rounding against a
 single-rounding discriminator; RoPE against rotation identities and an fp64
 rotation; mRoPE selection against three independent index formulas; KV scatter
-against permutation invariants.  The reference ships no golden vectors for
-this path.
+against permutation invariants; and, on the GPU, against the reference's own
+kernels built into oracle/_ref (tests/test_gpu_reference_kernels.py holds them to
+this restatement at the reference tests' allclose bar).  The reference ships no
+golden vectors for this path.
 """
 from __future__ import annotations
 
