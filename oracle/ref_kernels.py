@@ -75,11 +75,17 @@ def _section(section: Optional[Sequence[int]]):
     return None if section is None else (C.c_int64 * 3)(*section)
 
 
-def rope_rms(qkv, qw, kw, cos_sin, positions, T, hq, hk, hv, D, is_neox, eps, mrope_section=None, is_interleaved=False):
+def _in_range(index: torch.Tensor, bound: int) -> bool:
+    return int(index.min()) >= 0 and int(index.max()) < bound   # synchronises: skipped by timing loops (check_values=False)
+
+
+def rope_rms(qkv, qw, kw, cos_sin, positions, T, hq, hk, hv, D, is_neox, eps, mrope_section=None, is_interleaved=False,
+             check_values=True):
     """In place on qkv [T, hq+hk+hv, D].  positions [T] (rope) or [3, T] (mrope), int64, values below cos_sin's rows."""
     _bf16_cuda(qkv, qw, kw, cos_sin)
     assert qkv.numel() == T * (hq + hk + hv) * D and qw.numel() == D and kw.numel() == D and cos_sin.shape[-1] == D
-    assert positions.dtype == torch.int64 and positions.is_cuda and int(positions.max()) < cos_sin.shape[0] and int(positions.min()) >= 0
+    assert positions.dtype == torch.int64 and positions.is_cuda
+    assert not check_values or _in_range(positions, cos_sin.shape[0])
     if mrope_section is None:
         assert positions.dim() == 1 and positions.numel() == T
         ps0, ps1, n_axes = 0, positions.stride(0), 1
@@ -92,7 +98,7 @@ def rope_rms(qkv, qw, kw, cos_sin, positions, T, hq, hk, hv, D, is_neox, eps, mr
 
 
 def mrope_rms_set_kv(qkv, qw, kw, cos_sin, positions, T, hq, hk, hv, D, is_neox, eps, q, k_cache, v_cache, kv_loc,
-                     k_scale, v_scale, mrope_section=None, is_interleaved=False):
+                     k_scale, v_scale, mrope_section=None, is_interleaved=False, check_values=True):
     """positions [T] is passed as three equal rows (stride 0 over the axes) with one section covering D/2, which is
     how the reference's set_kv kernel does plain RoPE."""
     _bf16_cuda(qkv, qw, kw, cos_sin, q)
@@ -102,8 +108,8 @@ def mrope_rms_set_kv(qkv, qw, kw, cos_sin, positions, T, hq, hk, hv, D, is_neox,
     slots = k_cache.shape[0]
     assert k_cache.numel() == slots * hk * D and v_cache.numel() == slots * hv * D
     assert kv_loc.dtype == torch.int64 and kv_loc.is_cuda and kv_loc.numel() >= T
-    assert int(kv_loc.max()) < slots and int(kv_loc.min()) >= 0
-    assert positions.dtype == torch.int64 and positions.is_cuda and int(positions.max()) < cos_sin.shape[0] and int(positions.min()) >= 0
+    assert positions.dtype == torch.int64 and positions.is_cuda
+    assert not check_values or (_in_range(kv_loc[:T], slots) and _in_range(positions, cos_sin.shape[0]))
     if mrope_section is None:
         assert positions.dim() == 1 and positions.numel() == T
         ps0, ps1, section = 0, positions.stride(0), [D // 2, 0, 0]
