@@ -248,6 +248,20 @@ def main():
             for name, r in (("rope_kv_qwen3_T4096_us", workloads.config3()), ("mrope_kv_qwen2vl_T8192_us", workloads.config4())):
                 theirs, ours = ref_rope_us(r)
                 ref[name] = {"reference_kernel": theirs, "this_repository": ours}
+            # the two-stream op at the reference script's shape
+            B2, T0, T1, Hq2, Hk2, D2 = 2, 678, 3608, 24, 25, 128
+            g2 = torch.Generator(device=dev).manual_seed(7)
+            mk = lambda *shape: torch.randn(shape, device=dev, generator=g2).to(torch.bfloat16)
+            ins2 = [(mk(B2, T0, Hq2, D2), mk(B2, T0, Hk2, D2), mk(B2, T1, Hq2, D2), mk(B2, T1, Hk2, D2)) for _ in range(3)]
+            rest = [mk(D2) for _ in range(4)] + [mk(T0, D2), mk(T1, D2)]
+            outs2 = (torch.empty((B2, T0 + T1, Hq2, D2), dtype=torch.bfloat16, device=dev),
+                     torch.empty((B2, T0 + T1, Hk2, D2), dtype=torch.bfloat16, device=dev))
+            times = {}
+            for who, fn in (("reference_kernel", ref_kernels.rope_rms_2way), ("this_repository", capi.rope_rms_2way)):
+                times[who] = round(event_time_ms(lambda i=0: fn(*ins2[i % 3], *rest, B2, T0, T1, Hq2, Hk2, D2, False, 1e-6,
+                                                                *outs2), 50) * 1e3, 2)
+            ref["rope_2way_B2_678+3608_us"] = times
+            del ins2, outs2
             cpu_baseline["reference_kernels_on_this_gpu"] = ref
 
     # ------------------------------------------------------------------ secondary figures
