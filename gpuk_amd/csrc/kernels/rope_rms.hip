@@ -268,8 +268,11 @@ struct RopeUnit {
         u32x4 oa, ob;
         norm_rotate<T, D, NEOX>(xa, xb, wa, wb, cosv, sinv, a.eps, oa, ob);
 
+        // A negative slot marks a token that has no place in the cache (padding in a fixed-size decode batch): its Q
+        // row is still produced, its K and V rows are dropped.  The reference would write out of bounds.
+        const bool slot_ok = !SETKV || st.slot >= 0;  // wave-uniform
         const int head = st.head;
-        if (st.active) {
+        if (st.active && (st.is_q || slot_ok)) {
             if constexpr (!SETKV) {
                 uint16_t *dst = static_cast<uint16_t *>(a.qkv_out) + ((int64_t)st.t * heads_all + head) * D;
                 *reinterpret_cast<u32x4 *>(dst + c0(sub)) = oa;
@@ -300,7 +303,7 @@ struct RopeUnit {
             const float s = a.v_scale, rcp = 1.0f / s;
             const bool fast = scale_is_fast(s);
             u32x4 vchunk = st.vchunk;
-            for (int c = v_first; c < v_chunks; c += stride) {
+            for (int c = v_first; slot_ok && c < v_chunks; c += stride) {
                 if (c != v_first)
                     vchunk = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(st.token_in + (int64_t)heads_qk * D + 8 * c));
                 const int64_t off = st.slot * a.hv * D + 8 * (int64_t)c;
@@ -351,7 +354,9 @@ __global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
 
     if (h >= heads_qk) {  // a V head: only reached with a KV cache
         if constexpr (SETKV) {
-            const int64_t row = (a.kv_loc[t] * a.hv + (h - heads_qk)) * D;
+            const int64_t slot = a.kv_loc[t];
+            if (slot < 0) return;  // token without a cache slot
+            const int64_t row = (slot * a.hv + (h - heads_qk)) * D;
             for (int e = lane; e < D; e += 64) {
                 const float v = src[e];
                 if constexpr (KVFP8) {
@@ -400,7 +405,9 @@ __global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
     } else if (is_q) {
         dst = static_cast<float *>(a.q_out) + ((int64_t)t * a.hq + h) * D;
     } else {
-        const int64_t row = (a.kv_loc[t] * a.hk + (h - a.hq)) * D;
+        const int64_t slot = a.kv_loc[t];
+        if (slot < 0) return;  // token without a cache slot: nothing of a K head is kept
+        const int64_t row = (slot * a.hk + (h - a.hq)) * D;
         dst = static_cast<float *>(a.k_cache) + row;          // used when the cache is fp32
         dst8 = static_cast<uint8_t *>(a.k_cache) + row;       // used when it is fp8
     }

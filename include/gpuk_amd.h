@@ -114,7 +114,9 @@ int gpuk_rope_rms(void *qkv, const void *qw, const void *kw, const void *cos_sin
  *   q_out            : [num_tokens, hq, head_size] `dtype`, 16-byte aligned
  *   k_cache, v_cache : [slots, hk|hv, head_size]; `dtype` or e4m3fn bytes per kv_dtype; slots not named
  *                      by kv_loc are left bit-identical
- *   kv_loc           : [num_tokens] int64 slot per token (duplicates race; last writer wins)
+ *   kv_loc           : [num_tokens] int64 slot per token (duplicates race; last writer wins).  A negative slot
+ *                      marks a token with no place in the cache (padding): its q_out row is written, its K and V
+ *                      rows are dropped (an addition: the reference would write out of bounds)
  *   k_scale, v_scale : used only with GPUK_KV_E4M3FN: code = e4m3fn(rT(x / scale)), saturating at +-448
  */
 int gpuk_rope_rms_set_kv(const void *qkv, const void *qw, const void *kw, const void *cos_sin,

@@ -199,8 +199,11 @@ def rope_rms_set_kv_ref(
     if k_cache.dtype != qkv.dtype or scale_same_dtype_cache:
         k = k / k_scale
         v = v / v_scale
-    k_cache[kv_loc] = k.to(k_cache.dtype)
-    v_cache[kv_loc] = v.to(v_cache.dtype)
+    # a negative slot marks a token without a place in the cache (this build's extension; the reference's code would
+    # index out of range): its K and V are dropped
+    keep = kv_loc[:num_tokens] >= 0
+    k_cache[kv_loc[:num_tokens][keep]] = k.to(k_cache.dtype)[keep]
+    v_cache[kv_loc[:num_tokens][keep]] = v.to(v_cache.dtype)[keep]
     q_out.copy_(q.reshape(q_out.shape))
 
 

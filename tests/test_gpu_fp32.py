@@ -104,6 +104,7 @@ def test_rope_set_kv_fp32(device, kv_dtype, mrope):
     print(f"case fp32 rope set_kv cache={kv_dtype} mrope={mrope}", flush=True)
     T, hq, hk, hv, D = 45, 8, 2, 2, 128
     inp = rope_case(T, hq, hk, hv, D, True, 77, mrope, False, kv_dtype)
+    inp.kv_loc[3] = -1            # a padding token: q_out row written, K and V rows dropped
     qkv, qw, kw, cs, pos, loc = (t.to(device) for t in (inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, inp.kv_loc))
     k0, v0 = inp.new_cache()
     kc, vc = k0.to(device), v0.to(device)
@@ -121,7 +122,7 @@ def test_rope_set_kv_fp32(device, kv_dtype, mrope):
                           k_ref, v_ref, inp.kv_loc, inp.k_scale, inp.v_scale, inp.mrope_section, False)
     close32(q_out, q_ref, "q_out")
     kc, vc = kc.cpu(), vc.cpu()
-    sel = inp.kv_loc
+    sel = inp.kv_loc[inp.kv_loc >= 0]
     if kv_dtype == torch.float32:
         close32(kc[sel], k_ref[sel], "k rows")
         assert_bits_equal(vc[sel].view(torch.int32), v_ref[sel].view(torch.int32), "v rows")

@@ -316,3 +316,53 @@ def test_fp8_cache_saturates_out_of_range_values(device):
     assert not ((got_k.view(torch.uint8) & 0x7F) == 0x7F).any() and not ((got_v.view(torch.uint8) & 0x7F) == 0x7F).any()
     assert_codes_close(got_k, want_k, "saturated k codes")
     assert_bits_equal(got_v.view(torch.uint8), want_v.view(torch.uint8), "saturated v codes")
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_negative_slots_and_colliding_slots(device, fp8):
+    """kv_loc edge cases.  A negative slot (padding token) keeps q_out and drops the token's K and V rows; tokens that
+    name the same slot race, and the slot ends up holding exactly one of their rows."""
+    print(f"case kv_loc edge cases fp8={fp8}", flush=True)
+    inp = make(64, 8, 128, True, seed=123, fp8=fp8, hk=2, hv=2)
+    loc = inp.kv_loc.clone()
+    loc[5], loc[17], loc[63] = -1, -1, -7
+    inp.kv_loc = loc
+    check_set_kv_with_dropped = run_set_kv(inp, device)
+    q_out, kc, vc, (k0, v0) = check_set_kv_with_dropped
+    q_ref = torch.empty_like(q_out, device="cpu")
+    k_ref, v_ref = k0.clone(), v0.clone()
+    O.rope_rms_set_kv_ref(inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, 64, 8, 2, 2, 128, True, inp.eps, q_ref, k_ref,
+                          v_ref, loc, inp.k_scale, inp.v_scale)
+    assert_rotated_close(q_out, q_ref, "q_out with padded tokens")
+    raw = (lambda t: t.view(torch.uint8)) if fp8 else (lambda t: t.view(torch.int16))
+    kept = loc[loc >= 0]
+    untouched = torch.ones(inp.num_slots, dtype=torch.bool)
+    untouched[kept] = False
+    assert_bits_equal(raw(kc.cpu()[untouched]), raw(k0[untouched]), "slots no kept token names")
+    assert_bits_equal(raw(vc.cpu()[untouched]), raw(v0[untouched]), "slots no kept token names (v)")
+    (assert_codes_close if fp8 else assert_rotated_close)(kc.cpu()[kept], k_ref[kept], "K rows of the kept tokens")
+    assert_bits_equal(raw(vc.cpu()[kept]), raw(v_ref[kept]), "V rows of the kept tokens")
+
+    # collisions: tokens 0..7 all name slot 3
+    inp2 = make(64, 8, 128, True, seed=124, fp8=fp8, hk=2, hv=2)
+    loc2 = inp2.kv_loc.clone()
+    taken = set(loc2[8:].tolist())
+    shared = next(s for s in range(inp2.num_slots) if s not in taken)
+    loc2[:8] = shared
+    inp2.kv_loc = loc2
+    q_out, kc, vc, (k0, v0) = run_set_kv(inp2, device)
+    candidates_k, candidates_v = [], []
+    for t in range(8):   # the row each colliding token would write, from the oracle run with that token alone on the slot
+        k_one, v_one = k0.clone(), v0.clone()
+        only = loc2.clone()
+        only[:8] = -1
+        only[t] = shared
+        O.rope_rms_set_kv_ref(inp2.qkv, inp2.qw, inp2.kw, inp2.cos_sin, inp2.positions, 64, 8, 2, 2, 128, True, inp2.eps,
+                              torch.empty_like(q_out, device="cpu"), k_one, v_one, only, inp2.k_scale, inp2.v_scale)
+        candidates_k.append(k_one[shared])
+        candidates_v.append(v_one[shared])
+    got_v = raw(vc.cpu()[shared])
+    assert any(torch.equal(got_v, raw(c)) for c in candidates_v), "the shared slot holds one token's V row"
+    got_k = kc.cpu()[shared].float()
+    assert any(torch.allclose(got_k, c.float(), rtol=0.13 if fp8 else 1e-2, atol=5e-2) for c in candidates_k), \
+        "the shared slot holds one token's K row"
