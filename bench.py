@@ -373,6 +373,23 @@ def main():
                               "add_rmsnorm_quant_eager_us": round(event_time_ms(nq_call, 200) * 1e3, 2),
                               "rope_kv_fp8_eager_us": round(event_time_ms(rope_call, 200) * 1e3, 2)}
         extras["decode_us_per_call"] = decode
+        # static per-tensor quant at tokens=128, hidden=4096; scale = amax(normed)/448, taken once, outside the timing,
+        # from the same kernel's unquantised output
+        c1 = workloads.config1()
+        c1_g = c1.gamma.to(dev)
+        c1_normed = torch.empty((128, 4096), dtype=torch.bfloat16, device=dev)
+        capi.add_rmsnorm_quant(c1.x.to(dev), c1.residual.to(dev), c1_g, torch.empty_like(c1_normed), c1_normed, None, c1.eps, 0)
+        c1_scale = (c1_normed.float().abs().max() / 448.0).reshape(1)
+        c1_bufs = [(c1.x.to(dev).clone(), c1.residual.to(dev).clone(), torch.empty((128, 4096), dtype=torch.bfloat16, device=dev),
+                    torch.empty((128, 4096), dtype=torch.float8_e4m3fn, device=dev)) for _ in range(NG)]
+
+        def c1_call(i=0):
+            x, r_, ro, codes = c1_bufs[i % NG]
+            capi.add_rmsnorm_quant(x, r_, c1_g, ro, codes, c1_scale, c1.eps, 3)
+
+        extras["static_quant_T128_H4096_us_per_call"] = {"graph": round(graph_time_us(c1_call, NG), 2),
+                                                         "eager": round(event_time_ms(c1_call, 200) * 1e3, 2),
+                                                         "algorithmic_bytes": workloads.norm_quant_bytes(128, 4096, 3)}
         # the floor under those: a 1024-element increment kernel (one workgroup), same two ways of launching
         small = [torch.zeros(1024, dtype=torch.float32, device=dev) for _ in range(NG)]
 
