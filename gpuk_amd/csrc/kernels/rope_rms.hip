@@ -52,6 +52,9 @@ struct RopeArgs {
     float eps, k_scale, v_scale;
     // mRoPE: bit f of axis1 / axis2 set when rotary frequency f takes its position from axis 1 / 2
     uint32_t axis1[4], axis2[4];
+    // token-walking kernel: number of waves in the grid (token stride of a wave) and the token count
+    uint32_t walk_waves, num_tokens;
+    uint32_t walk_stream;  // 1: q_out / in-place stores (and in-place loads) bypass the L2; for large batches
 };
 
 // dword mask selecting the 16-bit halves whose bit is set in a 2-bit field
@@ -335,6 +338,449 @@ __global__ void __launch_bounds__(512) rope_rms_kernel(const RopeArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// Token-walking form for large batches.  A wave owns whole tokens (its first token is its wave index, the next one
+// walk_waves further on, ...) and walks each token's units in order.  What the one-wave-per-unit kernel above repeats
+// for every unit is done once per wave (norm weights unpacked to fp32) or once per token (position, slot, cos/sin row
+// loaded and unpacked), and the loads of the following kWalkRing units -- the first units of the wave's next token
+// included -- are in flight while the current one is finished, as is the next token's cos/sin row.  The grid is sized
+// to what the chip holds at once, so there is one dispatch round and no tail of partly filled rounds.
+//
+// Prefetched data travels global memory -> LDS directly (global_load_lds_dwordx4: lane l's 16 bytes land at
+// M0 + 16*l), so no register is the destination of a load in flight, and is waited for with an explicit
+// s_waitcnt vmcnt(N): left to the compiler, loop-carried load destinations get copied at every join (reading
+// registers whose data has not arrived) or the whole memory queue is drained at every step.  What makes the explicit
+// waits safe: N never exceeds the number of vector memory instructions issued after the transfer waited for (the
+// stores and loads the compiler emits only add to that number), vector memory instructions complete in issue order
+// on this target, and the LDS reads that follow a wait are ordinary loads the compiler orders after it (the wait
+// clobbers memory).  A staging buffer is refilled only after its previous content is in registers (in_registers()).
+constexpr int kWalkWaves = 4;  // waves per workgroup of the walking kernel
+constexpr int kWalkRing = 2;   // staging buffers per wave = units in flight beyond the current one
+
+template <bool NT>
+__device__ __forceinline__ void lds_fill16(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
+    if constexpr (NT) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(wave_base) : "memory");
+    } else {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(wave_base) : "memory");
+    }
+}
+// the same for lanes 0-31 only: 512 bytes of LDS
+__device__ __forceinline__ void lds_fill16_lanes32(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
+    uint64_t saved_exec;
+    asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_offset), "s"(wave_base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_fills() {  // until at most N vector memory instructions are outstanding
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// wait_fills<n> for a run-time, wave-uniform n; larger values wait as for kMaxBehind (waiting for more is always safe)
+constexpr int kMaxBehind = 16;
+__device__ __forceinline__ void wait_fills_upto(uint32_t n) {
+    switch (n) {
+#define GPUK_WAIT_CASE(N) case N: wait_fills<N>(); break;
+        GPUK_WAIT_CASE(0) GPUK_WAIT_CASE(1) GPUK_WAIT_CASE(2) GPUK_WAIT_CASE(3) GPUK_WAIT_CASE(4) GPUK_WAIT_CASE(5)
+        GPUK_WAIT_CASE(6) GPUK_WAIT_CASE(7) GPUK_WAIT_CASE(8) GPUK_WAIT_CASE(9) GPUK_WAIT_CASE(10) GPUK_WAIT_CASE(11)
+        GPUK_WAIT_CASE(12) GPUK_WAIT_CASE(13) GPUK_WAIT_CASE(14) GPUK_WAIT_CASE(15)
+#undef GPUK_WAIT_CASE
+        default: wait_fills<kMaxBehind>(); break;
+    }
+}
+// Pins the point by which a value read from LDS is in registers: the transfers that refill the same LDS bytes are
+// issued after this statement (both are volatile), so they cannot overtake the read.
+__device__ __forceinline__ void in_registers(u32x4 &v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ uint32_t lds_offset_of(const void *shared_ptr) { return (uint32_t)(uintptr_t)shared_ptr; }
+
+// A pair of 16-byte stores OFFSET bytes apart, streamed past the L2 (nt) or left to it.  The streaming form is
+// written in assembly: as two arms of a run-time choice, the compiler merges a non-temporal and a plain store into
+// one plain store.
+template <int OFFSET>
+__device__ __forceinline__ void store_pair(void *p, const u32x4 &a, const u32x4 &b, bool nt) {
+    if (nt) {
+        asm volatile("global_store_dwordx4 %0, %1, off nt\n\tglobal_store_dwordx4 %0, %2, off offset:%3 nt" ::"v"(p), "v"(a), "v"(b), "n"(OFFSET) : "memory");
+    } else {
+        *reinterpret_cast<u32x4 *>(p) = a;
+        *reinterpret_cast<u32x4 *>(static_cast<char *>(p) + OFFSET) = b;
+    }
+}
+// Same arithmetic as norm_rotate with the weights and the cos/sin values already unpacked to fp32.
+//   w[2j], w[2j+1]     : low / high half of dword j of the first chunk's weights;  w[8+2j], w[8+2j+1]: second chunk
+//   c[e], s[e]         : the lane's 8 cos / sin values in load_trig order
+template <typename T, int D, bool NEOX>
+__device__ __forceinline__ void norm_rotate_unpacked(const u32x4 &xa, const u32x4 &xb, const float (&w)[16],
+                                                     const float (&c)[8], const float (&s)[8], float eps, u32x4 &oa,
+                                                     u32x4 &ob) {
+    using P = Pack16<T>;
+    constexpr int LPH = D / 16;
+    float ss0 = 0.f, ss1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        ss0 = P::add_squares(xa[j], ss0);
+        ss1 = P::add_squares(xb[j], ss1);
+    }
+    const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
+    const float rstd = 1.0f / sqrtf(sumsq * (1.0f / D) + eps);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float a0 = P::round(w[2 * j] * P::round(P::lo(xa[j]) * rstd));
+        const float a1 = P::round(w[2 * j + 1] * P::round(P::hi(xa[j]) * rstd));
+        const float b0 = P::round(w[8 + 2 * j] * P::round(P::lo(xb[j]) * rstd));
+        const float b1 = P::round(w[8 + 2 * j + 1] * P::round(P::hi(xb[j]) * rstd));
+        if constexpr (NEOX) {
+            const float cl = c[2 * j], ch = c[2 * j + 1], sl = s[2 * j], sh = s[2 * j + 1];
+            oa[j] = P::pack(P::round(a0 * cl) - P::round(b0 * sl), P::round(a1 * ch) - P::round(b1 * sh));
+            ob[j] = P::pack(P::round(b0 * cl) + P::round(a0 * sl), P::round(b1 * ch) + P::round(a1 * sh));
+        } else {
+            oa[j] = P::pack(P::round(a0 * c[j]) - P::round(a1 * s[j]), P::round(a1 * c[j]) + P::round(a0 * s[j]));
+            ob[j] = P::pack(P::round(b0 * c[4 + j]) - P::round(b1 * s[4 + j]),
+                            P::round(b1 * c[4 + j]) + P::round(b0 * s[4 + j]));
+        }
+    }
+}
+
+template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
+struct RopeWalk {
+    using P = Pack16<T>;
+    static constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
+    enum Kind { kQ = 0, kK = 1, kMixed = 2 };
+
+    const RopeArgs &a;
+    const int lane, sub, hl;
+    const int heads_qk, heads_all, v_chunks;
+    float wq[16], wk[16];  // norm weights of the lane's two chunks, fp32
+    float c[8], s[8];      // cos / sin of the current token
+    int64_t slot;          // cache slot of the current token
+    uint32_t t, u;         // current token and unit
+
+    __device__ __forceinline__ RopeWalk(const RopeArgs &args, int lane_)
+        : a(args), lane(lane_), sub(lane_ % LPH), hl(lane_ / LPH), heads_qk(args.hq + args.hk),
+          heads_all(args.hq + args.hk + args.hv), v_chunks(SETKV ? args.hv * (D / 8) : 0) {}
+
+    __device__ __forceinline__ const uint16_t *token_row(uint32_t tt) const {
+        return static_cast<const uint16_t *>(a.qkv_in) + (int64_t)tt * heads_all * D;
+    }
+    __device__ __forceinline__ bool unit_has_v(uint32_t uu) const { return SETKV && (int)(uu * 64) < v_chunks; }
+
+    // Unit uu of token tt -> 2 KiB at LDS byte offset `stage`: the two 16-byte chunks of every lane (lanes past the
+    // last Q/K head re-read the last head).  Two transfers.
+    __device__ __forceinline__ void fill_unit(uint32_t stage, uint32_t tt, uint32_t uu) const {
+        const int head = min((int)(uu * HPW) + hl, heads_qk - 1);
+        const uint32_t off = (uint32_t)(head * D + 8 * sub) * 2u;
+        // streamed when the results go elsewhere; in place the same lines are written a moment later
+        // streamed when the results go elsewhere or the batch is large; in place and small, the same lines are
+        // written a moment later and are better kept
+        if (SETKV || a.walk_stream) {
+            lds_fill16<true>(stage, token_row(tt), off);
+            lds_fill16<true>(stage + 1024, token_row(tt), off + HALF * 2);
+        } else {
+            lds_fill16<false>(stage, token_row(tt), off);
+            lds_fill16<false>(stage + 1024, token_row(tt), off + HALF * 2);
+        }
+    }
+    // Unit uu's share of token tt's V row -> 1 KiB at `dst` (lanes past the row's end re-read its last chunk)
+    __device__ __forceinline__ void fill_v(uint32_t dst, uint32_t tt, uint32_t uu) const {
+        const int chunk = min((int)(uu * 64) + lane, v_chunks - 1);
+        lds_fill16<true>(dst, token_row(tt) + (int64_t)heads_qk * D, (uint32_t)chunk * 16u);
+    }
+    // Table row `pos` (2*D bytes: cos | sin) -> 512 bytes at `dst`, repeated 256/D times
+    __device__ __forceinline__ void fill_row(uint32_t dst, int64_t pos) const {
+        lds_fill16_lanes32(dst, static_cast<const uint16_t *>(a.cos_sin) + pos * D, (16u * lane) % (2u * D));
+    }
+    // Both weight vectors -> 1 KiB at `dst`: q weights in the first 512 bytes, k weights in the second
+    __device__ __forceinline__ void fill_weights(uint32_t dst) const {
+        const char *qw = static_cast<const char *>(a.qw), *kw = static_cast<const char *>(a.kw);
+        // one transfer with per-lane addresses relative to qw: lanes 32-63 reach over to kw
+        const int64_t k_minus_q = kw - qw;
+        const uint32_t within = (16u * (lane & 31)) % (2u * D);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(qw + (lane < 32 ? 0 : k_minus_q) + within) : "memory");
+    }
+    __device__ __forceinline__ void take_weights(const unsigned char *at) {
+        u32x4 qa = *reinterpret_cast<const u32x4 *>(at + 16 * sub), qb = *reinterpret_cast<const u32x4 *>(at + D + 16 * sub);
+        u32x4 ka = *reinterpret_cast<const u32x4 *>(at + 512 + 16 * sub), kb = *reinterpret_cast<const u32x4 *>(at + 512 + D + 16 * sub);
+        in_registers(qa);
+        in_registers(qb);
+        in_registers(ka);
+        in_registers(kb);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            wq[2 * j] = P::lo(qa[j]);
+            wq[2 * j + 1] = P::hi(qa[j]);
+            wq[8 + 2 * j] = P::lo(qb[j]);
+            wq[8 + 2 * j + 1] = P::hi(qb[j]);
+            wk[2 * j] = P::lo(ka[j]);
+            wk[2 * j + 1] = P::hi(ka[j]);
+            wk[8 + 2 * j] = P::lo(kb[j]);
+            wk[8 + 2 * j + 1] = P::hi(kb[j]);
+        }
+    }
+
+    // the staged rows (512 bytes each) -> c[], s[] of the current token
+    __device__ __forceinline__ void take_table(const unsigned char *rows, bool split) {
+        auto row_cos = [&](int r) -> u32x4 {
+            const unsigned char *p = rows + 512 * r;
+            if constexpr (NEOX) {
+                return *reinterpret_cast<const u32x4 *>(p + 16 * sub);
+            } else {
+                const u32x2 lo = *reinterpret_cast<const u32x2 *>(p + 8 * sub);
+                const u32x2 hi = *reinterpret_cast<const u32x2 *>(p + D / 2 + 8 * sub);
+                return u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+        };
+        auto row_sin = [&](int r) -> u32x4 {
+            const unsigned char *p = rows + 512 * r + D;
+            if constexpr (NEOX) {
+                return *reinterpret_cast<const u32x4 *>(p + 16 * sub);
+            } else {
+                const u32x2 lo = *reinterpret_cast<const u32x2 *>(p + 8 * sub);
+                const u32x2 hi = *reinterpret_cast<const u32x2 *>(p + D / 2 + 8 * sub);
+                return u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+        };
+        u32x4 cv = row_cos(0), sv = row_sin(0);
+        in_registers(cv);
+        in_registers(sv);
+        if constexpr (AXES == 3) {
+            if (split) {
+                u32x4 c1 = row_cos(1), s1 = row_sin(1), c2 = row_cos(2), s2 = row_sin(2);
+                in_registers(c1);
+                in_registers(s1);
+                in_registers(c2);
+                in_registers(s2);
+                const uint32_t b1 = trig_bits<D, NEOX>(a.axis1, sub), b2 = trig_bits<D, NEOX>(a.axis2, sub);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t m1 = halves_mask(b1 >> (2 * j)), m2 = halves_mask(b2 >> (2 * j));
+                    cv[j] = bitselect(m2, c2[j], bitselect(m1, c1[j], cv[j]));
+                    sv[j] = bitselect(m2, s2[j], bitselect(m1, s1[j], sv[j]));
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            c[2 * j] = P::lo(cv[j]);
+            c[2 * j + 1] = P::hi(cv[j]);
+            s[2 * j] = P::lo(sv[j]);
+            s[2 * j + 1] = P::hi(sv[j]);
+        }
+    }
+
+    // Norm, rotation and stores of the current unit.  Returns nothing; the caller counts the store instructions:
+    // two per kind of lane present (Q, K with a valid slot), one for the V chunk.
+    template <int KIND>
+    __device__ __forceinline__ void finish_unit(const u32x4 &xa, const u32x4 &xb, const u32x4 &v, bool has_v, bool stream_q) {
+        const int head_raw = (int)(u * HPW) + hl;
+        const bool active = KIND == kQ || head_raw < heads_qk;
+        const bool is_q = KIND == kQ || (KIND == kMixed && head_raw < a.hq);
+        u32x4 oa, ob;
+        if constexpr (KIND == kQ) {
+            norm_rotate_unpacked<T, D, NEOX>(xa, xb, wq, c, s, a.eps, oa, ob);
+        } else if constexpr (KIND == kK) {
+            norm_rotate_unpacked<T, D, NEOX>(xa, xb, wk, c, s, a.eps, oa, ob);
+        } else {
+            float w[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) w[i] = is_q ? wq[i] : wk[i];
+            norm_rotate_unpacked<T, D, NEOX>(xa, xb, w, c, s, a.eps, oa, ob);
+        }
+        const bool slot_ok = !SETKV || slot >= 0;  // wave-uniform; a negative slot drops the token's K and V rows
+        if constexpr (!SETKV) {
+            if (active) {
+                uint16_t *dst = static_cast<uint16_t *>(a.qkv_out) + ((int64_t)t * heads_all + head_raw) * D + 8 * sub;
+                store_pair<HALF * 2>(dst, oa, ob, stream_q);
+            }
+        } else {
+            if (KIND != kK && is_q) {
+                uint16_t *dst = static_cast<uint16_t *>(a.q_out) + ((int64_t)t * a.hq + head_raw) * D + 8 * sub;
+                store_pair<HALF * 2>(dst, oa, ob, stream_q);
+            }
+            if (KIND != kQ && !is_q && active && slot_ok) {
+                const int64_t row = (slot * a.hk + (head_raw - a.hq)) * D + 8 * sub;
+                if constexpr (KVFP8) {
+                    uint8_t *dst = static_cast<uint8_t *>(a.k_cache) + row;
+                    const float sc = a.k_scale, rcp = 1.0f / sc;
+                    if (scale_is_fast(sc)) {
+                        *reinterpret_cast<u32x2 *>(dst) = quantize_chunk<T, true>(oa, sc, rcp);
+                        *reinterpret_cast<u32x2 *>(dst + HALF) = quantize_chunk<T, true>(ob, sc, rcp);
+                    } else {
+                        *reinterpret_cast<u32x2 *>(dst) = quantize_chunk<T, false>(oa, sc, rcp);
+                        *reinterpret_cast<u32x2 *>(dst + HALF) = quantize_chunk<T, false>(ob, sc, rcp);
+                    }
+                } else {
+                    uint16_t *dst = static_cast<uint16_t *>(a.k_cache) + row;
+                    *reinterpret_cast<u32x4 *>(dst) = oa;
+                    *reinterpret_cast<u32x4 *>(dst + HALF) = ob;
+                }
+            }
+            // V: chunk u*64 + lane of the token's row, copied or quantised (the host takes this kernel only when
+            // the units of a token cover the whole row: units_per_token * 64 >= chunks)
+            const int chunk = (int)(u * 64) + lane;
+            if (has_v && slot_ok && chunk < v_chunks) {
+                const int64_t off = slot * a.hv * D + 8 * (int64_t)chunk;
+                if constexpr (!KVFP8) {
+                    *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(a.v_cache) + off) = v;
+                } else {
+                    const float sc = a.v_scale, rcp = 1.0f / sc;
+                    *reinterpret_cast<u32x2 *>(static_cast<uint8_t *>(a.v_cache) + off) =
+                        scale_is_fast(sc) ? quantize_chunk<T, true>(v, sc, rcp) : quantize_chunk<T, false>(v, sc, rcp);
+                }
+            }
+        }
+    }
+};
+
+template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
+__global__ void __launch_bounds__(kWalkWaves * 64)
+rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__restrict__ kv_loc, const RopeArgs a) {
+    using Walk = RopeWalk<T, D, NEOX, AXES, SETKV, KVFP8>;
+    constexpr int HPW = Walk::HPW, RING = kWalkRing;
+    __shared__ u32x4 s_stage[kWalkWaves][RING][128];  // per wave: the staged units, 2 KiB each
+    __shared__ u32x4 s_v[kWalkWaves][64];             // per wave: one unit's V chunks (first the norm weights)
+    __shared__ u32x4 s_rows[kWalkWaves][AXES * 32];   // per wave: the table rows of one token, 512 bytes each
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t first = blockIdx.x * kWalkWaves + wave;
+    const uint32_t n_waves = a.walk_waves, tokens = a.num_tokens, upt = a.units_per_token;
+    if (first >= n_waves) return;  // the host keeps walk_waves <= num_tokens
+    Walk w(a, threadIdx.x & 63);
+    w.t = first;
+    w.u = 0;
+    const uint32_t stage_at = lds_offset_of(&s_stage[wave][0][0]), v_at = lds_offset_of(&s_v[wave][0]),
+                   rows_at = lds_offset_of(&s_rows[wave][0]);
+
+    auto load_positions = [&](uint32_t tt, int64_t &p0, int64_t &p1, int64_t &p2) {
+        p0 = positions[(int64_t)tt * a.ps_token];
+        if constexpr (AXES == 3) {
+            p1 = positions[a.ps_axis + (int64_t)tt * a.ps_token];
+            p2 = positions[2 * a.ps_axis + (int64_t)tt * a.ps_token];
+        } else {
+            p1 = p2 = p0;
+        }
+    };
+    // `issued` counts the vector memory instructions this wave is known to have issued (transfers, and the stores
+    // of finished units); a mark is its value right after the transfers of one staged unit / V share / table row set.
+    // Waiting until at most issued - mark instructions are outstanding waits for exactly those transfers.
+    uint32_t issued = 0, rows_mark = 0, v_mark = 0;
+    uint32_t mark[RING];  // mark[0]: the current unit, mark[i]: the unit i further on
+    bool split = false;   // the three position axes of the token whose rows are staged differ
+    auto fill_table = [&](int64_t p0, int64_t p1, int64_t p2) {
+        w.fill_row(rows_at, p0);
+        issued += 1;
+        if constexpr (AXES == 3) {
+            split = p1 != p0 || p2 != p0;  // wave-uniform; text tokens carry three equal positions
+            if (split) {
+                w.fill_row(rows_at + 512, p1);
+                w.fill_row(rows_at + 1024, p2);
+                issued += 2;
+            }
+        }
+        rows_mark = issued;
+    };
+    // (ft, fu): the next unit to stage; fslot: the staging buffer it goes to
+    uint32_t ft = first, fu = 0, fslot = 0;
+    bool fmore = true;
+    auto stage_next = [&]() {
+        if (fmore) {
+            w.fill_unit(stage_at + fslot * 2048, ft, fu);
+            issued += 2;
+            if (++fu == upt) {
+                fu = 0;
+                ft += n_waves;
+                fmore = ft < tokens;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i + 1 < RING; ++i) mark[i] = mark[i + 1];
+        mark[RING - 1] = issued;
+        fslot = fslot + 1 == (uint32_t)RING ? 0 : fslot + 1;
+    };
+
+    // prologue.  The weights go first (they arrive soonest and are waited for first), then the first RING units,
+    // then what depends on the first token's positions.
+    w.fill_weights(v_at);
+    issued += 1;
+    const uint32_t weights_mark = issued;
+#pragma unroll
+    for (int i = 0; i < RING; ++i) mark[i] = 0;
+#pragma unroll
+    for (int i = 0; i < RING; ++i) stage_next();
+    // after the transfers above: a wait for these scalar loads placed ahead of them would hold them back
+    int64_t p0, p1, p2, np0 = 0, np1 = 0, np2 = 0;
+    load_positions(first, p0, p1, p2);
+    int64_t slot_next = SETKV ? kv_loc[first] : 0;
+    if (first + n_waves < tokens) load_positions(first + n_waves, np0, np1, np2);
+    fill_table(p0, p1, p2);
+    wait_fills_upto(issued - weights_mark);
+    w.take_weights(reinterpret_cast<const unsigned char *>(&s_v[wave][0]));  // before the V transfer below
+    if (w.unit_has_v(0)) {
+        w.fill_v(v_at, first, 0);
+        issued += 1;
+        v_mark = issued;
+    }
+
+    // One step: wait for the current unit's transfers (and, at a token's first unit, for its table rows), move it to
+    // registers, refill what that freed (next token's rows, next unit's V share, the unit RING ahead), finish the unit.
+    uint32_t cslot = 0;  // staging buffer of the current unit
+    const bool stream_q = a.walk_stream != 0;
+    for (;;) {
+        const bool cur_v = w.unit_has_v(w.u), token_start = w.u == 0;
+        uint32_t newest = mark[0];  // the newest transfer this step reads
+        if (cur_v) newest = max(newest, v_mark);
+        if (token_start) newest = max(newest, rows_mark);
+        wait_fills_upto(issued - newest);
+        const u32x4 *stage = &s_stage[wave][0][0] + cslot * 128;
+        u32x4 xa = stage[w.lane], xb = stage[64 + w.lane], v = u32x4{0, 0, 0, 0};
+        in_registers(xa);
+        in_registers(xb);
+        if (cur_v) {
+            v = s_v[wave][w.lane];
+            in_registers(v);
+        }
+        if (token_start) {
+            w.slot = slot_next;
+            w.take_table(reinterpret_cast<const unsigned char *>(&s_rows[wave][0]), split);
+            const uint32_t tn = w.t + n_waves;
+            if (tn < tokens) {
+                fill_table(np0, np1, np2);
+                if constexpr (SETKV) slot_next = kv_loc[tn];
+                if (tn + n_waves < tokens) load_positions(tn + n_waves, np0, np1, np2);
+            }
+        }
+        {   // the following unit's V share, before the unit RING ahead: a wait for it must not cover that one
+            uint32_t nu = w.u + 1, nt = w.t;
+            if (nu == upt) {
+                nu = 0;
+                nt += n_waves;
+            }
+            if (nt < tokens && w.unit_has_v(nu)) {
+                w.fill_v(v_at, nt, nu);
+                issued += 1;
+                v_mark = issued;
+            }
+        }
+        stage_next();  // refills the buffer just read; mark[0] now belongs to the following unit
+
+        const uint32_t h0 = w.u * HPW;
+        const bool slot_ok = !SETKV || w.slot >= 0;
+        if (h0 + HPW <= (uint32_t)a.hq) {
+            w.template finish_unit<Walk::kQ>(xa, xb, v, cur_v, stream_q);
+            issued += 2;
+        } else if (h0 >= (uint32_t)a.hq) {
+            w.template finish_unit<Walk::kK>(xa, xb, v, cur_v, stream_q);
+            issued += slot_ok ? 2 : 0;
+        } else {
+            w.template finish_unit<Walk::kMixed>(xa, xb, v, cur_v, stream_q);
+            issued += SETKV && slot_ok ? 4 : 2;  // in place one store sequence serves both kinds of lanes
+        }
+        if (SETKV && cur_v && slot_ok) issued += 1;
+        cslot = cslot + 1 == (uint32_t)RING ? 0 : cslot + 1;
+        if (++w.u == upt) {
+            w.u = 0;
+            w.t += n_waves;
+            if (w.t >= tokens) break;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // fp32 activations: the reference dispatches them through the same templates (src/ops/fused_rope.cpp:27-30, :108-111).
 // A compatibility path, not a tuned one: one wave per (token, head), lane l owns rotation pairs l, l+64, ...;
 // with a KV cache the V heads get waves of their own that copy or quantise.  Rounding to the activation type is the
@@ -584,9 +1030,41 @@ int launch_2way_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned ba
 }
 
 int g_block_threads = 0;    // 0 = default
+int g_walk = 0;             // token-walking kernel: 0 = built-in rule, 1 = never, 2 = always
+int g_walk_waves = 0;       // waves the walking grid may hold at once (0 = built-in)
+int g_walk_stream = 0;      // streaming stores of the walking kernel: 0 = built-in rule, 1 = never, 2 = always
+
+// Which kernel, measured on MI355X with D = 128 (32/8/8 and 28/4/4 heads, 16-bit cache, random slots):
+//   one wave per unit: best while all units fit the chip about once or twice (decode batches, T = 2048 x 72 heads);
+//   token-walking    : from about 20,000 units on; 18.6 against 20.3 us at T = 4096 x 40 heads, 28.1 against 31.2 us at
+//                      T = 8192 x 32 heads;
+//   streaming stores : q_out (or the in-place rows, then with streaming loads too) bypass the L2 once a call moves
+//                      more than the caches absorb: 34.5 against 41.0 us at T = 8192 x 40 heads (203 MB), 69.9 against
+//                      82.5 us at T = 16384, but 19.5 against 18.6 us at T = 4096 (102 MB) and no difference at 153 MB.
+constexpr int64_t kWalkMinUnits = 20000;
+constexpr int64_t kWalkStreamBytes = 176'000'000;
+constexpr uint32_t kWalkCapacity = 4096;  // waves the chip holds at once at 4 per SIMD: one dispatch round
 
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 int launch_one(const RopeArgs &a, hipStream_t stream) {
+    // the walking kernel shares a token's V row out over the token's units, one 16-byte chunk per lane and unit
+    const bool v_fits = !SETKV || (int64_t)a.units_per_token * 64 >= (int64_t)a.hv * (D / 8);
+    const bool walk = v_fits && (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits));
+    if (walk) {
+        // every wave the same number of tokens (the last ones one fewer)
+        const uint32_t capacity = g_walk_waves ? (uint32_t)g_walk_waves : kWalkCapacity;
+        const uint32_t tokens_per_wave = (a.num_tokens + capacity - 1) / capacity;
+        RopeArgs b = a;
+        b.walk_waves = (a.num_tokens + tokens_per_wave - 1) / tokens_per_wave;
+        // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
+        const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
+        const int64_t walk_bytes = SETKV ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
+                                               (KVFP8 ? 1 : 2) * ((int64_t)a.num_tokens * a.hk * D + elems_v)
+                                         : 4 * elems_qk;
+        b.walk_stream = g_walk_stream == 2 || (g_walk_stream == 0 && walk_bytes >= kWalkStreamBytes) ? 1u : 0u;
+        rope_rms_walk_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<(b.walk_waves + kWalkWaves - 1) / kWalkWaves, kWalkWaves * 64, 0, stream>>>(a.positions, a.kv_loc, b);
+        return hip_status(hipGetLastError());
+    }
     const int threads = g_block_threads ? g_block_threads : 256;
     const uint32_t units_per_block = threads / 64;
     const uint32_t blocks = (a.total_units + units_per_block - 1) / units_per_block;
@@ -718,6 +1196,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     a.v_cache = v_cache;
     a.kv_loc = kv_loc;
     a.total_units = (uint32_t)(upt * T);
+    a.num_tokens = (uint32_t)T;
     a.units_per_token = (uint32_t)upt;
     a.upt_magic = upt == 1 ? 0u : (uint32_t)(((1ull << 32) + (uint64_t)upt - 1) / (uint64_t)upt);
     a.hq = (int)hq;
@@ -736,6 +1215,9 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
 
 void set_rope_tuning(int key, int value) {
     if (key == 0) g_block_threads = value;
+    if (key == 1) g_walk = value;
+    if (key == 2) g_walk_waves = value;
+    if (key == 3) g_walk_stream = value;
 }
 
 }  // namespace gpuk

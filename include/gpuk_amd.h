@@ -114,7 +114,8 @@ int gpuk_rope_rms(void *qkv, const void *qw, const void *kw, const void *cos_sin
  *   q_out            : [num_tokens, hq, head_size] `dtype`, 16-byte aligned
  *   k_cache, v_cache : [slots, hk|hv, head_size]; `dtype` or e4m3fn bytes per kv_dtype; slots not named
  *                      by kv_loc are left bit-identical
- *   kv_loc           : [num_tokens] int64 slot per token (duplicates race; last writer wins).  A negative slot
+ *   kv_loc           : [num_tokens] int64 slot per token.  Tokens that name the same slot race: every aligned group of
+ *                      8 elements of the slot's K and V rows comes whole from one of them, the rows may mix.  A negative slot
  *                      marks a token with no place in the cache (padding): its q_out row is written, its K and V
  *                      rows are dropped (an addition: the reference would write out of bounds)
  *   k_scale, v_scale : used only with GPUK_KV_E4M3FN: code = e4m3fn(rT(x / scale)), saturating at +-448
@@ -163,10 +164,11 @@ int gpuk_increment_floats(float *data, int64_t n, void *stream);
 
 /* Launch-shape knobs for sweeps and for the tests that show the results do not depend on them; value 0 restores
  * the built-in choice.  Keys: "norm_quant_nchunk" (1/2/4/8 16-byte chunks per lane), "norm_quant_threads" (lanes
- * per row), "norm_quant_rows" (1 or 2 rows per workgroup), "norm_quant_paired_stores" (0/1), "norm_quant_lds_pad"
- * (bytes of idle LDS per workgroup), "norm_quant_row_group_shift" (log2 of the run of consecutive rows one XCD takes;
- * -1, not 0, restores the built-in rule), "rope_block_threads" (64/128/256/512).  Unknown keys or values return
- * GPUK_ERR_INVALID_ARG.  Not part of the reference. */
+ * per row), "norm_quant_row_group_shift" (log2 of the run of consecutive rows one XCD takes; -1, not 0, restores the
+ * built-in rule), "rope_block_threads" (64/128/256/512, one-wave-per-unit kernel), "rope_walk" (token-walking kernel:
+ * 1 never, 2 always), "rope_walk_waves" (waves of its grid), "rope_walk_stream" (its streaming stores: 1 never,
+ * 2 always).  Unknown keys or values return GPUK_ERR_INVALID_ARG.  The settings are process-global plain variables
+ * read at launch: set them from one thread while no other thread is launching.  Not part of the reference. */
 int gpuk_set_tuning(const char *key, int value);
 
 #ifdef __cplusplus

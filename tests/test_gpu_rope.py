@@ -186,6 +186,68 @@ def test_launch_shape_variants(device, threads):
         capi.set_tuning("rope_block_threads", 0)
 
 
+WALK_CASES = [
+    # tokens, (hq, hk, hv), head size, neox, mrope, interleaved, fp8
+    (45, (32, 8, 8), 128, True, False, False, False),     # whole units of Q heads, one of K heads
+    (61, (28, 4, 4), 128, True, True, False, False),      # a unit that mixes Q and K heads; three position axes
+    (37, (20, 20, 20), 64, False, True, True, True),      # 16 heads per unit, GPT-J pairs, fp8 cache
+    (29, (9, 3, 3), 256, True, True, True, False),        # 4 heads per unit, a partly filled last unit
+    (33, (64, 8, 8), 128, False, False, False, True),     # nine units per token, GPT-J pairs, fp8 cache
+    (19, (3, 2, 1), 128, True, False, False, False),      # a single, partly filled unit per token
+    (23, (7, 2, 0), 128, True, False, False, False),      # no V heads
+]
+
+
+@pytest.mark.parametrize("case", range(len(WALK_CASES)))
+@pytest.mark.parametrize("waves", [0, 5, 1])
+@pytest.mark.parametrize("stream", [1, 2])
+def test_token_walking_kernel(device, case, waves, stream):
+    """Large batches run a second kernel in which a wave walks the units of whole tokens with the following units'
+    loads in flight.  Forced onto small batches here: as many waves as tokens, five waves, and a single wave that
+    walks every token; stores through the L2 and streamed past it.  Its arithmetic is the one-wave-per-unit
+    kernel's, so besides meeting the oracle the two must agree bit for bit."""
+    from gpuk_amd import capi
+
+    tokens, heads, hs, neox, mrope, interleaved, fp8 = WALK_CASES[case]
+    print(f"case walk {WALK_CASES[case]} waves={waves} stream={stream}", flush=True)
+    inp = make(tokens, heads[0], hs, neox, seed=900 + case, mrope=mrope, interleaved=interleaved, fp8=fp8, hk=heads[1],
+               hv=heads[2])
+    if case == 0:   # two padding tokens
+        inp.kv_loc[3], inp.kv_loc[tokens - 1] = -1, -5
+    nqk = heads[0] + heads[1]
+    capi.set_tuning("rope_walk", 1)
+    try:
+        base_set = run_set_kv(inp, device)
+        base_inplace = run_inplace(inp, device)
+        capi.set_tuning("rope_walk", 2)
+        capi.set_tuning("rope_walk_waves", waves)
+        capi.set_tuning("rope_walk_stream", stream)
+        got_set = run_set_kv(inp, device)
+        got_inplace = run_inplace(inp, device)
+    finally:
+        capi.set_tuning("rope_walk", 0)
+        capi.set_tuning("rope_walk_waves", 0)
+        capi.set_tuning("rope_walk_stream", 0)
+    raw = lambda t: t.cpu().contiguous().view(torch.uint8)
+    for name, a, b in zip(("q_out", "k_cache", "v_cache"), got_set[:3], base_set[:3]):
+        assert torch.equal(raw(a), raw(b)), f"{name}: the two kernels differ"
+    assert torch.equal(raw(got_inplace), raw(base_inplace)), "in place: the two kernels differ"
+    if case != 0:
+        check_set_kv(inp, got_set, f"[walk {case}]")
+    want = oracle_inplace(inp)
+    assert_rotated_close(got_inplace[:, :nqk], want[:, :nqk], "in place q,k")
+    assert_bits_equal(got_inplace[:, nqk:], want[:, nqk:], "in place v")
+
+
+def test_kernel_choice_by_batch_size(device):
+    """The built-in rule: small batches take the one-wave-per-unit kernel, large ones the walking kernel; with too
+    many V heads for the walking kernel's sharing-out of the V row the first one runs whatever the size.  All of
+    them meet the oracle (sizes on both sides of the switch)."""
+    for tokens, heads in ((3900, (32, 8, 8)), (4100, (32, 8, 8)), (20100, (4, 4, 10))):
+        inp = make(tokens, heads[0], 128, True, seed=tokens, hk=heads[1], hv=heads[2])
+        check_set_kv(inp, run_set_kv(inp, device), f"[T={tokens} heads={heads}]")
+
+
 @pytest.mark.parametrize("hq,hk,hv,head_size", [(3, 1, 40, 64), (1, 1, 17, 256), (7, 2, 0, 128), (2, 9, 33, 128)])
 def test_value_heads_outnumber_the_waves(device, hq, hk, hv, head_size):
     """The V row is shared out over the waves that rotate Q and K; with few Q/K heads and many V heads each wave
@@ -321,7 +383,7 @@ def test_fp8_cache_saturates_out_of_range_values(device):
 @pytest.mark.parametrize("fp8", [False, True])
 def test_negative_slots_and_colliding_slots(device, fp8):
     """kv_loc edge cases.  A negative slot (padding token) keeps q_out and drops the token's K and V rows; tokens that
-    name the same slot race, and the slot ends up holding exactly one of their rows."""
+    name the same slot race: every 8-element piece of the slot's rows comes whole from one of them."""
     print(f"case kv_loc edge cases fp8={fp8}", flush=True)
     inp = make(64, 8, 128, True, seed=123, fp8=fp8, hk=2, hv=2)
     loc = inp.kv_loc.clone()
@@ -361,8 +423,15 @@ def test_negative_slots_and_colliding_slots(device, fp8):
                               torch.empty_like(q_out, device="cpu"), k_one, v_one, only, inp2.k_scale, inp2.v_scale)
         candidates_k.append(k_one[shared])
         candidates_v.append(v_one[shared])
-    got_v = raw(vc.cpu()[shared])
-    assert any(torch.equal(got_v, raw(c)) for c in candidates_v), "the shared slot holds one token's V row"
-    got_k = kc.cpu()[shared].float()
-    assert any(torch.allclose(got_k, c.float(), rtol=0.13 if fp8 else 1e-2, atol=5e-2) for c in candidates_k), \
-        "the shared slot holds one token's K row"
+    # What the kernel guarantees for a shared slot: every 8-element piece (one lane's store: 16 bytes of a 16-bit
+    # cache, 8 bytes of an fp8 cache) comes whole from one of the colliding tokens.  Different pieces of the row are
+    # written by different store instructions and waves, so the row as a whole may mix tokens.
+    got_v = raw(vc.cpu()[shared]).reshape(-1, 8)
+    cand_v = torch.stack([raw(c).reshape(-1, 8) for c in candidates_v])            # [8 tokens, pieces, 8]
+    v_from_a_token = (cand_v == got_v[None]).all(dim=-1).any(dim=0)
+    assert bool(v_from_a_token.all()), f"V pieces not from any colliding token: {(~v_from_a_token).nonzero().flatten().tolist()}"
+    got_k = kc.cpu()[shared].float().reshape(-1, 8)
+    cand_k = torch.stack([c.float().reshape(-1, 8) for c in candidates_k])
+    rtol = 0.13 if fp8 else 1e-2
+    k_close = ((cand_k - got_k[None]).abs() <= 5e-2 + rtol * cand_k.abs()).all(dim=-1).any(dim=0)
+    assert bool(k_close.all()), f"K pieces not from any colliding token: {(~k_close).nonzero().flatten().tolist()}"
