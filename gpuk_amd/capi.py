@@ -14,7 +14,8 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libgpuk_amd.so")
 
 EXPORTS = ("gpuk_status_string", "gpuk_abi_version", "gpuk_add_rmsnorm_quant", "gpuk_rope_rms",
-           "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_increment_floats", "gpuk_set_tuning")
+           "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_increment_floats", "gpuk_set_tuning",
+           "gpuk_add_rmsnorm_quant_traffic_only", "gpuk_add_rmsnorm_quant_launch_shape")
 
 DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 QUANT_NONE, QUANT_FP8_DYNAMIC, QUANT_FP8_E4M3FNUZ, QUANT_FP8_STATIC = 0, 1, 2, 3
@@ -55,6 +56,10 @@ def lib():
                                                                              C.c_void_p, C.c_void_p, C.c_void_p]
         L.gpuk_increment_floats.restype = C.c_int
         L.gpuk_increment_floats.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
+        L.gpuk_add_rmsnorm_quant_traffic_only.restype = C.c_int
+        L.gpuk_add_rmsnorm_quant_traffic_only.argtypes = [C.c_void_p] * 5 + [C.c_int64, C.c_int64, C.c_void_p]
+        L.gpuk_add_rmsnorm_quant_launch_shape.restype = C.c_int
+        L.gpuk_add_rmsnorm_quant_launch_shape.argtypes = [C.c_int64, C.c_int64, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.gpuk_copy_bytes.restype = C.c_int
         L.gpuk_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
         _lib = L
@@ -85,6 +90,23 @@ def add_rmsnorm_quant(x, residual_in, gamma, residual_out, norm_out, scale, eps:
                                       _stream(stream))
     if rc:
         raise GpukError(rc, "gpuk_add_rmsnorm_quant")
+
+
+def add_rmsnorm_quant_traffic_only(x, residual_in, residual_out, codes, scale, stream=None) -> None:
+    tokens = x.numel() // x.shape[-1]
+    rc = lib().gpuk_add_rmsnorm_quant_traffic_only(_ptr(x), _ptr(residual_in), _ptr(residual_out), _ptr(codes), _ptr(scale),
+                                                   tokens, x.shape[-1], _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_add_rmsnorm_quant_traffic_only")
+
+
+def add_rmsnorm_quant_launch_shape(tokens: int, hidden: int, dtype=torch.bfloat16):
+    """(lanes per row, 16-byte chunks per lane) of the launch gpuk_add_rmsnorm_quant makes for this batch."""
+    lanes, chunks = C.c_int(0), C.c_int(0)
+    rc = lib().gpuk_add_rmsnorm_quant_launch_shape(tokens, hidden, DTYPE[dtype], C.byref(lanes), C.byref(chunks))
+    if rc:
+        raise GpukError(rc, "gpuk_add_rmsnorm_quant_launch_shape")
+    return lanes.value, chunks.value
 
 
 def _pos_args(positions):

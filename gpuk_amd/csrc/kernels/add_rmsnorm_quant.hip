@@ -43,19 +43,33 @@ __device__ __forceinline__ bool scale_in_fast_range(float s) {
     return s >= 0x1p-60f && s <= 0x1p60f;
 }
 
-// ROWS: token rows a workgroup handles side by side (their loads are all in flight together and their two
-// reductions share the barriers).  PAIRED: lanes 2k and 2k+1 swap half of their codes so that every lane issues one
-// 16-byte store per two chunks instead of two 8-byte stores (needs NCHUNK even and an even number of chunks per row).
-template <typename T, int NCHUNK, int QUANT, bool PAIRED, int ROWS>
+// max(m, |a|, |b|) in one instruction.  Written in assembly: the inputs come out of integer-typed conversions and
+// the compiler turns fabs() of such a value into a separate v_and instead of a source modifier.  NaNs are dropped
+// (callers track them apart).
+__device__ __forceinline__ float max3_abs(float m, float a, float b) {
+    float r;
+    asm("v_max3_f32 %0, |%1|, |%2|, %3" : "=v"(r) : "v"(a), "v"(b), "v"(m));
+    return r;
+}
+
+// a / b for finite a and b > 0 comfortably normal, given rcp = RN(1/b): the correctly rounded quotient by one
+// multiply and two fused multiply-adds (Markstein), arranged so that a = -0 gives -0: with e = q*b - a the last step
+// fma(-e, rcp, q) adds two negative zeros, where the usual fma(a - q*b, rcp, q) adds +0 and -0.
+__device__ __forceinline__ float div_by_rcp_finite(float a, float b, float rcp) {
+    const float q = a * rcp;
+    const float e = __builtin_fmaf(q, b, -a);
+    return __builtin_fmaf(-e, rcp, q);
+}
+
+template <typename T, int NCHUNK, int QUANT>
 __global__ void __launch_bounds__(kMaxThreads)
-add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ residual_in,
-                       const u32x4 *__restrict__ gamma, u32x4 *__restrict__ residual_out,
-                       void *__restrict__ norm_out, float *__restrict__ scale_io, int tokens, int chunks_per_row,
-                       float hidden_f, float rcp_hidden, float eps, float fp8_max, int group_shift, int remap_end) {
+add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
+                       const u32x4 *__restrict__ gamma, u32x4 *residual_out, void *norm_out,
+                       float *__restrict__ scale_io, int tokens, int chunks_per_row, float hidden_f, float rcp_hidden,
+                       int hidden_pow2, float eps, float fp8_max, int group_shift, int remap_end) {
     using P = Pack16<T>;
-    static_assert(!PAIRED || NCHUNK % 2 == 0, "paired code stores need an even chunk count per lane");
-    __shared__ float s_sum[ROWS * kReduceSlots];
-    __shared__ float s_max[ROWS * kReduceSlots];
+    __shared__ float s_sum[kReduceSlots];
+    __shared__ float s_max[kReduceSlots];
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
@@ -63,37 +77,27 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
     // Workgroup ids are handed to the 8 XCDs round-robin.  Below remap_end the rows are dealt out in runs of
     // 2^group_shift consecutive rows per XCD instead of one row each (which rows run concurrently stays the same;
     // which XCD's L2 and fabric port each row goes through changes).
-    int wg = blockIdx.x;
-    if (wg < remap_end) {
-        const int xcd = wg & 7, idx = wg >> 3;
-        wg = ((((idx >> group_shift) << 3) | xcd) << group_shift) | (idx & ((1 << group_shift) - 1));
+    int row = blockIdx.x;
+    if (row < remap_end) {
+        const int xcd = row & 7, idx = row >> 3;
+        row = ((((idx >> group_shift) << 3) | xcd) << group_shift) | (idx & ((1 << group_shift) - 1));
     }
-    const int row0 = wg * ROWS;
+    const int64_t row_base = (int64_t)row * chunks_per_row;
 
-    // ---- phase 0: issue every load of the rows before touching any of them.  A row past the end re-reads the
-    // last row (its results are never stored), so the loads need no row predicate.
-    u32x4 xv[ROWS][NCHUNK], rv[ROWS][NCHUNK], gv[NCHUNK];
+    // ---- phase 0: issue every load of the row before touching any of them.  The row is loaded whole before any of
+    // it is stored, so residual_out may be the same buffer as residual_in or x.
+    u32x4 xv[NCHUNK], rv[NCHUNK], gv[NCHUNK];
     bool live[NCHUNK];
-    int64_t row_base[ROWS];
-    bool row_ok[ROWS];
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        row_ok[r] = row0 + r < tokens;
-        row_base[r] = (int64_t)min(row0 + r, tokens - 1) * chunks_per_row;
-    }
 #pragma unroll
     for (int i = 0; i < NCHUNK; ++i) {
         const int c = i * nthreads + tid;
         live[i] = c < chunks_per_row;
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            if (live[i]) {
-                xv[r][i] = load_stream(x + row_base[r] + c);
-                rv[r][i] = load_stream(residual_in + row_base[r] + c);
-            } else {
-                xv[r][i] = u32x4{0, 0, 0, 0};
-                rv[r][i] = u32x4{0, 0, 0, 0};
-            }
+        if (live[i]) {
+            xv[i] = load_stream(x + row_base + c);
+            rv[i] = load_stream(residual_in + row_base + c);
+        } else {
+            xv[i] = u32x4{0, 0, 0, 0};
+            rv[i] = u32x4{0, 0, 0, 0};
         }
     }
 #pragma unroll
@@ -105,140 +109,138 @@ add_rmsnorm_quant_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ re
     // ---- phase 1: res = rT(x + r), stored once; sum of squares of the *rounded* residual.  Waves in this phase
     // are given issue priority over the arithmetic of phases 2-3 so that their residual stores leave early (+0.4 %).
     __builtin_amdgcn_s_setprio(1);
-    float sumsq[ROWS];
+    float ss0 = 0.f, ss1 = 0.f;
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        float ss0 = 0.f, ss1 = 0.f;
+    for (int i = 0; i < NCHUNK; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t w = P::pack(P::lo(xv[i][j]) + P::lo(rv[i][j]), P::hi(xv[i][j]) + P::hi(rv[i][j]));
+            xv[i][j] = w;  // xv now holds the residual
+            if (j & 1) ss1 = P::add_squares(w, ss1);
+            else ss0 = P::add_squares(w, ss0);
+        }
+        if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+    }
+    float sumsq[1] = {ss0 + ss1};
+    block_allreduce<SumOp, 1>(sumsq, s_sum, num_waves);
+    __builtin_amdgcn_s_setprio(0);
+
+    // ---- phase 2: n2 = rT(gamma * rT(res * rstd)); row amax for the dynamic scale.
+    // mean = sumsq / H as an exact IEEE quotient: a multiplication when H is a power of two (exact, and rounded like
+    // the quotient when the result is subnormal), a division otherwise
+    const float mean = hidden_pow2 ? sumsq[0] * rcp_hidden : sumsq[0] / hidden_f;
+    const float rstd = 1.0f / sqrtf(mean + eps);
+    if constexpr (QUANT == GPUK_QUANT_NONE) {
+        u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base;
 #pragma unroll
         for (int i = 0; i < NCHUNK; ++i) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t w = P::pack(P::lo(xv[r][i][j]) + P::lo(rv[r][i][j]), P::hi(xv[r][i][j]) + P::hi(rv[r][i][j]));
-                xv[r][i][j] = w;  // xv now holds the residual
-                if (j & 1) ss1 = P::add_squares(w, ss1);
-                else ss0 = P::add_squares(w, ss0);
+                const float lo = P::lo(gv[i][j]) * P::round(P::lo(xv[i][j]) * rstd);
+                const float hi = P::hi(gv[i][j]) * P::round(P::hi(xv[i][j]) * rstd);
+                xv[i][j] = P::pack(lo, hi);  // xv now holds the normed row
             }
-            if (live[i] && row_ok[r]) store_stream(residual_out + row_base[r] + i * nthreads + tid, xv[r][i]);
-        }
-        sumsq[r] = ss0 + ss1;
-    }
-    block_allreduce<SumOp, ROWS>(sumsq, s_sum, num_waves);
-
-    __builtin_amdgcn_s_setprio(0);
-    // ---- phase 2: n2 = rT(gamma * rT(res * rstd)); row amax for the dynamic scale
-    float amax[ROWS];
-    float nv[ROWS][QUANT == GPUK_QUANT_NONE ? 1 : NCHUNK][8];
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        // mean = sumsq / H as an exact IEEE quotient: by the reciprocal of H (computed on the host) while that is
-        // safe, by a division otherwise
-        const float mean = (sumsq[r] >= 0x1p-60f && sumsq[r] <= 0x1p100f) ? div_by_rcp(sumsq[r], hidden_f, rcp_hidden)
-                                                                         : sumsq[r] / hidden_f;
-        const float rstd = 1.0f / sqrtf(mean + eps);
-        if constexpr (QUANT == GPUK_QUANT_NONE) {
-#pragma unroll
-            for (int i = 0; i < NCHUNK; ++i) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float lo = P::lo(gv[i][j]) * P::round(P::lo(xv[r][i][j]) * rstd);
-                    const float hi = P::hi(gv[i][j]) * P::round(P::hi(xv[r][i][j]) * rstd);
-                    xv[r][i][j] = P::pack(lo, hi);  // xv now holds the normed row
-                }
-            }
-            amax[r] = 0.f;
-        } else {
-            // the normed row stays in fp32 registers, every value already rounded to the 16-bit type
-            // fmax drops NaNs where the reference's amax propagates them: they are tracked apart
-            float m0 = 0.f, m1 = 0.f;
-            bool any_nan = false;
-#pragma unroll
-            for (int i = 0; i < NCHUNK; ++i) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float lo = P::round(P::lo(gv[i][j]) * P::round(P::lo(xv[r][i][j]) * rstd));
-                    const float hi = P::round(P::hi(gv[i][j]) * P::round(P::hi(xv[r][i][j]) * rstd));
-                    nv[r][i][2 * j] = lo;
-                    nv[r][i][2 * j + 1] = hi;
-                    if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
-                        if (j & 1) m1 = __builtin_fmaxf(m1, __builtin_fmaxf(__builtin_fabsf(lo), __builtin_fabsf(hi)));
-                        else m0 = __builtin_fmaxf(m0, __builtin_fmaxf(__builtin_fabsf(lo), __builtin_fabsf(hi)));
-                        any_nan |= __builtin_isunordered(lo, hi);
-                    }
-                }
-            }
-            amax[r] = any_nan ? __builtin_nanf("") : __builtin_fmaxf(m0, m1);
-        }
-    }
-
-    if constexpr (QUANT == GPUK_QUANT_NONE) {
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base[r];
-#pragma unroll
-            for (int i = 0; i < NCHUNK; ++i)
-                if (live[i] && row_ok[r]) store_stream(out + i * nthreads + tid, xv[r][i]);
+            if (live[i]) store_stream(out + i * nthreads + tid, xv[i]);
         }
         return;
     } else {
-        if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) block_allreduce<MaxOp, ROWS>(amax, s_max, num_waves);
+        // the normed row stays in fp32 registers, every value already rounded to the 16-bit type.
+        // v_max3_f32 drops NaNs where the reference's amax propagates them: they are tracked apart
+        float nv[NCHUNK][8];
+        float m0 = 0.f, m1 = 0.f;
+        bool any_nan = false;
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            float scale;
-            if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
-                scale = amax[r] == 0.f ? 1.f : amax[r] / fp8_max;
-                if (tid == 0 && row_ok[r]) scale_io[row0 + r] = scale;
-            } else {
-                scale = scale_io[0];
-            }
-
-            // ---- phase 3: code = e4m3fn(clamp(n2 / scale)), 8 codes per chunk.  With the dynamic scale
-            // |n2 / scale| <= 448 * (1 + 2^-23), which the converter already rounds to 448: no clamp needed.
-            constexpr bool kClamp = QUANT != GPUK_QUANT_FP8_DYNAMIC;
-            uint8_t *out = reinterpret_cast<uint8_t *>(norm_out) + row_base[r] * 8;
-            if (__builtin_expect(scale_in_fast_range(scale), 1)) {
-                const float rcp = 1.0f / scale;
-                auto encode = [&](const float (&v)[8]) {
-                    float q[8];
+        for (int i = 0; i < NCHUNK; ++i) {
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        q[j] = div_by_rcp(v[j], scale, rcp);
-                    }
-                    if constexpr (kClamp) clamp8_sym(q, fp8_max);
-                    return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
-                };
-                if constexpr (PAIRED) {
-                    const bool odd = tid & 1;
-#pragma unroll
-                    for (int i = 0; i < NCHUNK; i += 2) {
-                        const u32x2 c0 = encode(nv[r][i]), c1 = encode(nv[r][i + 1]);
-                        // the even lane keeps iteration i and sends i+1; the odd lane the other way round
-                        const u32x2 keep = odd ? c1 : c0, send = odd ? c0 : c1;
-                        const u32x2 recv = {dpp_xor1_u32(send[0]), dpp_xor1_u32(send[1])};
-                        const u32x4 both = odd ? u32x4{recv[0], recv[1], keep[0], keep[1]}
-                                               : u32x4{keep[0], keep[1], recv[0], recv[1]};
-                        const int c = odd ? (i + 1) * nthreads + tid - 1 : i * nthreads + tid;  // first chunk of the pair
-                        if (c < chunks_per_row && row_ok[r]) store_stream(reinterpret_cast<u32x4 *>(out + (int64_t)c * 8), both);
-                    }
-                } else {
-#pragma unroll
-                    for (int i = 0; i < NCHUNK; ++i) {
-                        const u32x2 codes = encode(nv[r][i]);
-                        if (live[i] && row_ok[r]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
-                    }
-                }
-            } else {
-                // scale so small or large that its reciprocal leaves the normal range: plain IEEE division
-                // (unrolled like the fast path: a runtime index into the register arrays would move them to LDS)
-#pragma unroll
-                for (int i = 0; i < NCHUNK; ++i) {
-                    float q[8];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) q[j] = clamp_sym(nv[r][i][j] / scale, fp8_max);
-                    const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
-                    if (live[i] && row_ok[r]) store_stream(reinterpret_cast<u32x2 *>(out) + i * nthreads + tid, codes);
+            for (int j = 0; j < 4; ++j) {
+                const float lo = P::round(P::lo(gv[i][j]) * P::round(P::lo(xv[i][j]) * rstd));
+                const float hi = P::round(P::hi(gv[i][j]) * P::round(P::hi(xv[i][j]) * rstd));
+                nv[i][2 * j] = lo;
+                nv[i][2 * j + 1] = hi;
+                if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
+                    if (j & 1) m1 = max3_abs(m1, lo, hi);
+                    else m0 = max3_abs(m0, lo, hi);
+                    any_nan |= __builtin_isunordered(lo, hi);
                 }
             }
         }
+        float scale;
+        if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
+            float amax[1] = {any_nan ? __builtin_nanf("") : __builtin_fmaxf(m0, m1)};
+            block_allreduce<MaxOp, 1>(amax, s_max, num_waves);
+            scale = amax[0] == 0.f ? 1.f : amax[0] / fp8_max;
+            if (tid == 0) scale_io[row] = scale;
+        } else {
+            scale = scale_io[0];
+        }
+
+        // ---- phase 3: code = e4m3fn(clamp(n2 / scale)), 8 codes per chunk.  With the dynamic scale every value is
+        // finite and |n2 / scale| <= 448 * (1 + 2^-23), which the converter already rounds to 448: no clamp, and the
+        // short form of the quotient.  The static scale may meet anything: clamp, and the form that restores what a
+        // division gives for infinite and NaN numerators.
+        constexpr bool kDynamic = QUANT == GPUK_QUANT_FP8_DYNAMIC;
+        u32x2 *out = reinterpret_cast<u32x2 *>(norm_out) + row_base;
+        if (__builtin_expect(scale_in_fast_range(scale), 1)) {
+            const float rcp = 1.0f / scale;
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i) {
+                float q[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) q[j] = kDynamic ? div_by_rcp_finite(nv[i][j], scale, rcp) : div_by_rcp(nv[i][j], scale, rcp);
+                if constexpr (!kDynamic) clamp8_sym(q, fp8_max);
+                const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                if (live[i]) store_stream(out + i * nthreads + tid, codes);
+            }
+        } else {
+            // scale so small or large (or not a number) that its reciprocal leaves the normal range: plain IEEE
+            // division (unrolled like the fast path: a runtime index into the register arrays would move them to LDS)
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i) {
+                float q[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) q[j] = clamp_sym(nv[i][j] / scale, fp8_max);
+                const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                if (live[i]) store_stream(out + i * nthreads + tid, codes);
+            }
+        }
+    }
+}
+
+// Calibration: the memory traffic of add_rmsnorm_quant_rows without its arithmetic.  Same launch shape, lane-to-chunk
+// mapping, row-to-workgroup mapping, streaming loads and stores and the same two workgroup barriers; the "residual"
+// is x ^ r and the "codes" fold it to half its size.  What this kernel reaches is the ceiling of the access pattern.
+template <int NCHUNK>
+__global__ void __launch_bounds__(kMaxThreads)
+add_rmsnorm_quant_traffic_only(const u32x4 *x, const u32x4 *residual_in, u32x4 *residual_out, u32x2 *codes,
+                               float *__restrict__ scale_out, int chunks_per_row, int group_shift, int remap_end) {
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    int row = blockIdx.x;
+    if (row < remap_end) {
+        const int xcd = row & 7, idx = row >> 3;
+        row = ((((idx >> group_shift) << 3) | xcd) << group_shift) | (idx & ((1 << group_shift) - 1));
+    }
+    const int64_t row_base = (int64_t)row * chunks_per_row;
+    u32x4 xv[NCHUNK], rv[NCHUNK];
+    bool live[NCHUNK];
+#pragma unroll
+    for (int i = 0; i < NCHUNK; ++i) {
+        const int c = i * nthreads + tid;
+        live[i] = c < chunks_per_row;
+        xv[i] = live[i] ? load_stream(x + row_base + c) : u32x4{0, 0, 0, 0};
+        rv[i] = live[i] ? load_stream(residual_in + row_base + c) : u32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int i = 0; i < NCHUNK; ++i) {
+        xv[i] ^= rv[i];
+        if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+    }
+    __syncthreads();
+    __syncthreads();
+    if (tid == 0) scale_out[row] = 1.0f;
+#pragma unroll
+    for (int i = 0; i < NCHUNK; ++i) {
+        const u32x2 folded = {xv[i][0] + xv[i][1], xv[i][2] + xv[i][3]};
+        if (live[i]) store_stream(codes + row_base + i * nthreads + tid, folded);
     }
 }
 
@@ -383,15 +385,13 @@ add_rmsnorm_quant_f32_rows(const f32x4 *__restrict__ x, const f32x4 *__restrict_
 
 int g_force_nchunk = 0;   // 0 = heuristic; set through gpuk_set_tuning for sweeps
 int g_force_threads = 0;  // 0 = heuristic
-int g_rows = 0;           // rows per workgroup: 0 = heuristic, 1 or 2
 int g_row_group_shift = -1;  // -1 = heuristic, else log2 of the run of consecutive rows an XCD takes (0 = one row)
-int g_lds_pad = 0;        // unused dynamic LDS bytes per workgroup: caps the workgroups resident per CU
-int g_paired = 0;         // 16-byte paired code stores (measured no faster than 8-byte stores; kept selectable)
 
 // Lanes per row and chunks per lane.  Measured on MI355X over rows of 1024 .. 16384 elements: two chunks per lane
 // on as many lanes as that needs (up to 1024) streams best or ties everywhere (1-6 % over one or four chunks per
-// lane), unless rounding up to whole waves would idle more lanes that way; longer rows double the chunks per lane; few rows (decode) spread each row over as many lanes as possible
-// to shorten the dependent load -> reduce -> reduce -> store chain.
+// lane), unless rounding up to whole waves would idle more lanes that way; longer rows double the chunks per lane;
+// few rows (decode) spread each row over as many lanes as possible to shorten the dependent
+// load -> reduce -> reduce -> store chain.
 void pick_shape(int64_t tokens, int chunks_per_row, int *threads, int *nchunk) {
     auto fits = [&](int n) { return (int64_t)n * kMaxThreads >= chunks_per_row; };
     int n;
@@ -433,31 +433,25 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
         add_rmsnorm_quant_long_rows<T, QUANT><<<grid, kMaxThreads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale, chunks, hf, eps, fp8_max);
         return hip_status(hipGetLastError());
     }
-    const bool paired = g_paired && QUANT != GPUK_QUANT_NONE && nchunk % 2 == 0 && chunks % 2 == 0;
-    // two rows per workgroup once there are enough rows to keep every CU busy with half as many workgroups
-    const int rows = g_rows ? g_rows : 1;  // two rows per workgroup measured slower at every shape tried
-    const dim3 grid2((unsigned)((tokens + rows - 1) / rows));
     const float rcp_hidden = 1.0f / hf;
+    const int hidden_pow2 = (hidden & (hidden - 1)) == 0;
     const int tok = (int)tokens;
     // Runs of 64 rows per XCD: measured +1.1 % for 16 KiB rows (8192 rows); neutral or 1-10 % slower for every other
     // row size tried (2, 3, 4, 8, 10, 14, 32 KiB) and for fewer rows, hence the narrow rule.
     const int64_t row_bytes = hidden * 2;
-    int group_shift = row_bytes == 16384 && grid2.x >= 1024 ? 6 : 0;
+    int group_shift = row_bytes == 16384 && tokens >= 1024 ? 6 : 0;
     if (g_row_group_shift >= 0) group_shift = g_row_group_shift;
-    const int remap_end = group_shift > 0 ? (int)((grid2.x >> (3 + group_shift)) << (3 + group_shift)) : 0;
-#define GPUK_LAUNCH_NQ(N, PAIRED, ROWS)                                                                       \
-    add_rmsnorm_quant_rows<T, N, QUANT, PAIRED, ROWS><<<grid2, threads, g_lds_pad, stream>>>(xs, rs, gs, ro, norm_out, scale, tok, \
-                                                                                    chunks, hf, rcp_hidden, eps, fp8_max, group_shift, remap_end)
-#define GPUK_LAUNCH_NQ_ROWS(N, PAIRED) \
-    if (rows == 2) GPUK_LAUNCH_NQ(N, PAIRED, 2); else GPUK_LAUNCH_NQ(N, PAIRED, 1)
+    const int remap_end = group_shift > 0 ? (int)((tokens >> (3 + group_shift)) << (3 + group_shift)) : 0;
+#define GPUK_LAUNCH_NQ(N)                                                                                         \
+    add_rmsnorm_quant_rows<T, N, QUANT><<<grid, threads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale, tok, chunks, hf, \
+                                                                      rcp_hidden, hidden_pow2, eps, fp8_max, group_shift, remap_end)
     switch (nchunk) {
-        case 1: GPUK_LAUNCH_NQ_ROWS(1, false); break;
-        case 2: if (paired) { GPUK_LAUNCH_NQ_ROWS(2, true); } else { GPUK_LAUNCH_NQ_ROWS(2, false); } break;
-        case 4: if (paired) { GPUK_LAUNCH_NQ_ROWS(4, true); } else { GPUK_LAUNCH_NQ_ROWS(4, false); } break;
-        case 8: if (paired) GPUK_LAUNCH_NQ(8, true, 1); else GPUK_LAUNCH_NQ(8, false, 1); break;
+        case 1: GPUK_LAUNCH_NQ(1); break;
+        case 2: GPUK_LAUNCH_NQ(2); break;
+        case 4: GPUK_LAUNCH_NQ(4); break;
+        case 8: GPUK_LAUNCH_NQ(8); break;
         default: return GPUK_ERR_INTERNAL;
     }
-#undef GPUK_LAUNCH_NQ_ROWS
 #undef GPUK_LAUNCH_NQ
     return hip_status(hipGetLastError());
 }
@@ -510,13 +504,54 @@ int launch_quant(int quant_mode, const void *x, const void *residual_in, const v
 void set_norm_quant_tuning(int key, int value) {
     if (key == 0) g_force_nchunk = value;
     if (key == 1) g_force_threads = value;
-    if (key == 2) g_paired = value;
-    if (key == 3) g_rows = value;
-    if (key == 4) g_lds_pad = value;
     if (key == 5) g_row_group_shift = value;
 }
 
 }  // namespace gpuk
+
+extern "C" int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *residual_in, void *residual_out,
+                                                   void *codes, float *scale, int64_t tokens, int64_t hidden,
+                                                   void *stream) {
+    using namespace gpuk;
+    if (tokens <= 0 || hidden <= 0 || hidden % 8 != 0 || tokens > 0x7fffffffLL) return GPUK_ERR_INVALID_ARG;
+    if (!x || !residual_in || !residual_out || !codes || !scale) return GPUK_ERR_INVALID_ARG;
+    if (!aligned16(x) || !aligned16(residual_in) || !aligned16(residual_out) || !aligned8(codes)) return GPUK_ERR_MISALIGNED;
+    const int chunks = (int)(hidden / 8);
+    int threads, nchunk;
+    pick_shape(tokens, chunks, &threads, &nchunk);
+    if (nchunk == 0) return GPUK_ERR_UNSUPPORTED;  // rows that do not stay in registers
+    int group_shift = hidden * 2 == 16384 && tokens >= 1024 ? 6 : 0;
+    if (g_row_group_shift >= 0) group_shift = g_row_group_shift;
+    const int remap_end = group_shift > 0 ? (int)((tokens >> (3 + group_shift)) << (3 + group_shift)) : 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    auto xs = static_cast<const u32x4 *>(x), rs = static_cast<const u32x4 *>(residual_in);
+    auto ro = static_cast<u32x4 *>(residual_out);
+    auto co = static_cast<u32x2 *>(codes);
+    const dim3 grid((unsigned)tokens);
+    switch (nchunk) {
+        case 1: add_rmsnorm_quant_traffic_only<1><<<grid, threads, 0, s>>>(xs, rs, ro, co, scale, chunks, group_shift, remap_end); break;
+        case 2: add_rmsnorm_quant_traffic_only<2><<<grid, threads, 0, s>>>(xs, rs, ro, co, scale, chunks, group_shift, remap_end); break;
+        case 4: add_rmsnorm_quant_traffic_only<4><<<grid, threads, 0, s>>>(xs, rs, ro, co, scale, chunks, group_shift, remap_end); break;
+        default: add_rmsnorm_quant_traffic_only<8><<<grid, threads, 0, s>>>(xs, rs, ro, co, scale, chunks, group_shift, remap_end); break;
+    }
+    return hip_status(hipGetLastError());
+}
+
+extern "C" int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidden, int dtype, int *lanes_per_row,
+                                                   int *chunks_per_lane) {
+    using namespace gpuk;
+    if (tokens <= 0 || hidden <= 0 || !lanes_per_row || !chunks_per_lane) return GPUK_ERR_INVALID_ARG;
+    const int elems = dtype == GPUK_DTYPE_F32 ? 4 : 8;
+    if (hidden % elems != 0) return GPUK_ERR_UNSUPPORTED;
+    if (dtype == GPUK_DTYPE_F32) {  // the fp32 path sweeps the row: lanes only
+        const int want = ((int)(hidden / 4) + 63) / 64 * 64;
+        *lanes_per_row = want < kMaxThreads ? want : kMaxThreads;
+        *chunks_per_lane = 0;
+        return GPUK_OK;
+    }
+    pick_shape(tokens, (int)(hidden / 8), lanes_per_row, chunks_per_lane);
+    return GPUK_OK;
+}
 
 extern "C" int gpuk_add_rmsnorm_quant(const void *x, const void *residual_in, const void *gamma, void *residual_out,
                                       void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps,

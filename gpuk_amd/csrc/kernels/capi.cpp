@@ -30,23 +30,9 @@ extern "C" int gpuk_set_tuning(const char *key, int value) {
         gpuk::set_norm_quant_tuning(1, value);
         return GPUK_OK;
     }
-    if (strcmp(key, "norm_quant_lds_pad") == 0) {
-        if (value < 0 || value > 65536) return GPUK_ERR_INVALID_ARG;
-        gpuk::set_norm_quant_tuning(4, value);
-        return GPUK_OK;
-    }
     if (strcmp(key, "norm_quant_row_group_shift") == 0) {  // -1 = heuristic, 0..10
         if (value < -1 || value > 10) return GPUK_ERR_INVALID_ARG;
         gpuk::set_norm_quant_tuning(5, value);
-        return GPUK_OK;
-    }
-    if (strcmp(key, "norm_quant_rows") == 0) {
-        if (value < 0 || value > 2) return GPUK_ERR_INVALID_ARG;
-        gpuk::set_norm_quant_tuning(3, value);
-        return GPUK_OK;
-    }
-    if (strcmp(key, "norm_quant_paired_stores") == 0) {
-        gpuk::set_norm_quant_tuning(2, value != 0);
         return GPUK_OK;
     }
     if (strcmp(key, "rope_walk") == 0) {

@@ -15,8 +15,6 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 
-constexpr int DPP_QUAD_XOR1_CTRL = 0xB1;  // quad_perm [1,0,3,2]
-
 struct BF16 {};  // tag types: the 16-bit storage format of activations
 struct FP16 {};
 
@@ -63,23 +61,6 @@ template <> struct Pack16<FP16> {
         return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
     }
 };
-
-// Running maximum of |value| over packed 16-bit floats, kept as two u16 magnitudes in one dword: for
-// non-NaN values the magnitude bits order like the values, so one v_and + one v_pk_max_u16 serve two elements.
-typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t absmax_packed(uint32_t acc, uint32_t w) {
-    const u16x2_t a = __builtin_bit_cast(u16x2_t, acc), b = __builtin_bit_cast(u16x2_t, w & 0x7fff7fffu);
-    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
-}
-template <typename T>
-__device__ __forceinline__ float absmax_to_float(uint32_t acc) {
-    const uint32_t lo = acc & 0xffffu, hi = acc >> 16;
-    return Pack16<T>::from_bits16(lo > hi ? lo : hi);
-}
-
-__device__ __forceinline__ uint32_t dpp_xor1_u32(uint32_t v) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, DPP_QUAD_XOR1_CTRL, 0xf, 0xf, true);
-}
 
 // ---- DPP lane exchange.  CTRL encodings: quad_perm[a,b,c,d] = a|b<<2|c<<4|d<<6,
 // row_half_mirror = 0x141, row_mirror = 0x140 (both reverse within 8 / 16 lanes).

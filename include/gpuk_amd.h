@@ -76,6 +76,9 @@ int gpuk_abi_version(void);
  *                                  all_reduce_fusion_impl.h:389-401)
  *   fp8_max                      : clamp bound and amax divisor; 448 (OCP e4m3fn) or 240 (the
  *                                  reference's fp8e4m3fn::max_value, src/common/float8.h:216-218)
+ *
+ * residual_out may be the same buffer as residual_in or as x (the usual in-place residual stream): every row is read
+ * whole before any of it is written.  Partial overlap, and norm_out overlapping an input, are not allowed.
  */
 int gpuk_add_rmsnorm_quant(const void *x, const void *residual_in, const void *gamma, void *residual_out,
                            void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps, int dtype,
@@ -154,6 +157,24 @@ int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1, const voi
  * Counterpart of the reference's micro-benchmark test/cpp/global_memory_bandwidth.cpp:95-114.
  */
 int gpuk_copy_bytes(void *dst, const void *src, int64_t nbytes, void *stream);
+
+/*
+ * Roofline calibration: the memory traffic of gpuk_add_rmsnorm_quant (16-bit activations, fp8 output, per-token
+ * scale) without its arithmetic: same launch shape, lane-to-data mapping, streaming loads and stores and barriers;
+ * residual_out receives x ^ residual_in, codes a fold of it, scale 1.0 per token.  Its duration is the ceiling of the
+ * access pattern, to be read beside the real kernel's.  x, residual_in, residual_out: [tokens, hidden] 16-bit;
+ * codes: [tokens, hidden] bytes; scale: [tokens] fp32; hidden a multiple of 8 and at most 65536.
+ * Not part of the reference (its micro-benchmarks are test/cpp/global_memory_bandwidth.cpp).
+ */
+int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *residual_in, void *residual_out, void *codes,
+                                        float *scale, int64_t tokens, int64_t hidden, void *stream);
+
+/*
+ * The launch shape gpuk_add_rmsnorm_quant picks for a batch: lanes per token row (= workgroup size; one workgroup
+ * per row) and 16-byte chunks per lane (0: rows too long for registers, swept three times).  For reports.
+ */
+int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidden, int dtype, int *lanes_per_row,
+                                        int *chunks_per_lane);
 
 /*
  * Launch-cost calibration: data[i] += 1 for i in [0, n) (data 16-byte aligned).  With a small n the call costs

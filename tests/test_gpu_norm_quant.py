@@ -154,20 +154,18 @@ def test_every_chunking_variant(device, nchunk):
         capi.set_tuning("norm_quant_nchunk", 0)
 
 
-@pytest.mark.parametrize("threads,nchunk,paired,rows", [(512, 2, 1, 1), (512, 2, 0, 2), (256, 4, 1, 2), (1024, 2, 1, 1),
-                                                        (128, 8, 1, 1), (448, 2, 1, 2), (1024, 1, 0, 2), (256, 4, 0, 1)])
-def test_launch_shape_variants(device, threads, nchunk, paired, rows):
-    """Workgroup size, chunks per lane, rows per workgroup and the paired 16-byte code stores are tuning choices only."""
+@pytest.mark.parametrize("threads,nchunk", [(512, 2), (256, 4), (1024, 2), (128, 8), (448, 2), (1024, 1), (1024, 8)])
+def test_launch_shape_variants(device, threads, nchunk):
+    """Workgroup size and chunks per lane are tuning choices only."""
     from gpuk_amd import capi
 
-    print(f"case variants threads={threads} nchunk={nchunk} paired={paired} rows={rows}", flush=True)
+    print(f"case variants threads={threads} nchunk={nchunk}", flush=True)
     capi.set_tuning("norm_quant_nchunk", nchunk)
     capi.set_tuning("norm_quant_threads", threads)
-    capi.set_tuning("norm_quant_paired_stores", paired)
-    capi.set_tuning("norm_quant_rows", rows)
     try:
-        for hidden in (8192, 7168, 1032):
-            inp = workloads.norm_quant_inputs(301, hidden, seed=threads + hidden, res_sigma=2.0, outlier_frac=0.01)
+        for hidden in (8192, 7168, 1032) + ((40960,) if nchunk == 8 else ()):
+            inp = workloads.norm_quant_inputs(301 if hidden < 40960 else 37, hidden, seed=threads + hidden, res_sigma=2.0,
+                                              outlier_frac=0.01)
             for quant in (0, 1, 3):
                 st = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
                 check(inp, quant, run_capi(inp, quant, device, static_scale=st), static_scale=st,
@@ -175,8 +173,44 @@ def test_launch_shape_variants(device, threads, nchunk, paired, rows):
     finally:
         capi.set_tuning("norm_quant_nchunk", 0)
         capi.set_tuning("norm_quant_threads", 0)
-        capi.set_tuning("norm_quant_paired_stores", 0)
-        capi.set_tuning("norm_quant_rows", 0)
+
+
+@pytest.mark.parametrize("alias", ["residual_in", "x"])
+@pytest.mark.parametrize("quant", [0, 1, 3])
+def test_residual_out_may_alias_an_input(device, alias, quant):
+    """The in-place residual stream: residual_out is the same buffer as residual_in (or as x).  Every row is read
+    whole before any of it is stored, so the results are those of separate buffers."""
+    from gpuk_amd import capi
+
+    for tokens, hidden in ((300, 8192), (37, 40960), (5, 7168), (3, 65536 + 64)):
+        print(f"case alias={alias} quant={quant} {tokens}x{hidden}", flush=True)
+        inp = workloads.norm_quant_inputs(tokens, hidden, seed=hidden + quant, res_sigma=2.0, outlier_frac=0.01)
+        static = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
+        x, r, g = inp.x.to(device), inp.residual.to(device), inp.gamma.to(device)
+        norm = torch.empty((tokens, hidden), dtype=torch.bfloat16 if quant == 0 else torch.float8_e4m3fn, device=device)
+        scale = None if quant == 0 else (torch.empty((tokens, 1), dtype=torch.float32, device=device) if quant == 1
+                                         else static.to(device).float().reshape(1))
+        res_out = r if alias == "residual_in" else x
+        capi.add_rmsnorm_quant(x, r, g, res_out, norm, scale, inp.eps, quant)
+        torch.cuda.synchronize()
+        check(inp, quant, (res_out, norm, scale), static_scale=static, tag=f"[alias {alias} {tokens}x{hidden} q{quant}]")
+
+
+def test_negative_zero_keeps_its_sign(device):
+    """A zero residual under a negative gamma norms to -0, whose quotient by the scale is -0 and whose code is 0x80:
+    the short form of the quotient used with the dynamic scale must not turn it into +0."""
+    inp = workloads.norm_quant_inputs(9, 4096, seed=77, res_sigma=1.0)
+    inp.gamma[::3] = -inp.gamma[::3]
+    inp.residual[:, 100:400] = -inp.x[:, 100:400]       # exact zeros in the residual
+    inp.x[4], inp.residual[4] = 0, 0                      # an all-zero row
+    for quant in (1, 3):
+        static = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
+        res, norm, scale = run_capi(inp, quant, device, static_scale=static)
+        res_ref, norm_ref, scale_ref = O.add_rmsnorm_quant_ref(inp.x, inp.residual, inp.gamma, inp.eps, quant, static_scale=static)
+        want = norm_ref.view(torch.uint8)
+        assert int((want[:, 100:400] == 0x80).sum()) > 500, "the case must contain negative zeros"
+        assert torch.equal(norm.cpu().view(torch.uint8)[:, 100:400], want[:, 100:400]), f"quant {quant}: codes of the zero columns"
+        assert_codes_close(norm, norm_ref, f"[neg zero q{quant}]")
 
 
 @pytest.mark.parametrize("shift", [-1, 0, 1, 3, 6, 7])
