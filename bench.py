@@ -9,10 +9,11 @@ cache can serve a repeat.  Prints ONE JSON line:
 
   value      achieved HBM GB/s over the K timed steps = algorithmic bytes (7*T*H + 4*T + 2*H) / wall time
   roofline   the same kernel timed per launch with HIP events on the launch stream, against 8 TB/s
-  cpu_baseline  the restated torch reference on the host's cores, on a bounded row sample of the same batch; where
-             oracle/_ref was built, also the reference's own kernels timed on this GPU beside this repository's
-  extras     secondary figures: copy-kernel ceiling, the RoPE + KV-write kernel on its two configurations,
-             decode-shape latencies (us/call)
+  cpu_baseline  the restated torch reference on the host's cores on the same batch (at least 3 calls, about 10 s);
+             where oracle/_ref was built, also the reference's own kernels timed on this GPU beside this repository's
+  extras     secondary figures: copy-kernel ceiling, the fused kernel's traffic without its arithmetic, the RoPE +
+             KV-write kernel on its two configurations with a plain copy of the same bytes beside each, decode-shape
+             latencies (us/call)
 """
 from __future__ import annotations
 
@@ -41,15 +42,30 @@ def parse_args():
     ap.add_argument("--hidden", type=int, default=8192)
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the batch the CPU baseline runs on")
-    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU time budget of the baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the batch the CPU baseline runs on (0 = all of them)")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU time budget of the baseline leg (at least 3 calls are made)")
     return ap.parse_args()
 
 
-def event_time_ms(fn, iters, warmup=3):
+def settle_clocks(fn, ms=30.0):
+    """Runs fn(i) untimed for `ms` milliseconds: after an idle spell (the CPU leg, buffer set-up) the GPU's clocks take
+    some tens of milliseconds to come back up, which a short timed loop would otherwise measure."""
+    import torch
+
+    t0, n = time.perf_counter(), 0
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(10):
+            fn(n)
+            n += 1
+        torch.cuda.synchronize()
+
+
+def event_time_ms(fn, iters, warmup=3, settle_ms=30.0):
     """Average duration of fn() in ms from HIP events on the current stream (where fn launches)."""
     import torch
 
+    if settle_ms > 0:
+        settle_clocks(fn, settle_ms)
     for _ in range(warmup):
         fn()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -93,8 +109,7 @@ def graph_time_us(call, n_in_graph=20, replays=30):
     with torch.cuda.graph(g):
         for i in range(n_in_graph):
             call(i)
-    for _ in range(3):
-        g.replay()
+    settle_clocks(lambda i: g.replay(), 20.0)
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     a.record()
@@ -174,10 +189,13 @@ def main():
     avg_ms = ev0.elapsed_time(ev1) / args.steps
     _, med_ms, min_ms = per_launch_ms(step, min(args.steps, 200))
     achieved = alg_bytes / (avg_ms * 1e-3) / 1e9
+    lanes, chunks = capi.add_rmsnorm_quant_launch_shape(T, H, torch.bfloat16)
+    profiled = (T, H) == (8192, 8192)   # the counter runs behind the committed traffic figure used this shape
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": traffic_from_profile("add_rmsnorm_quant_8192x8192.md"),
-                "kernel": "add_rmsnorm_quant_rows<BF16, 2 chunks/lane, dynamic> (8192 workgroups x 512 lanes)",
+                "traffic": traffic_from_profile("add_rmsnorm_quant_8192x8192.md") if profiled else None,
+                "kernel": (f"add_rmsnorm_quant_rows<BF16, {chunks} chunks/lane, dynamic> ({T} workgroups x {lanes} lanes)"
+                           if chunks else f"add_rmsnorm_quant_long_rows<BF16, dynamic> ({T} workgroups x {lanes} lanes)"),
                 "avg_launch_us": round(avg_ms * 1e3, 2),
                 "single_launch_median_us": round(med_ms * 1e3, 2), "single_launch_min_us": round(min_ms * 1e3, 2),
                 "algorithmic_bytes": alg_bytes}
@@ -187,7 +205,7 @@ def main():
     if not args.no_cpu:
         from oracle import torch_oracle as O
 
-        rows = min(args.cpu_rows, T)
+        rows = min(args.cpu_rows, T) if args.cpu_rows > 0 else T
         ncores = os.cpu_count() or 1
         threads = int(os.environ.get("OMP_NUM_THREADS", ncores))
         torch.set_num_threads(threads)
@@ -202,7 +220,8 @@ def main():
         t_med = sorted(times)[len(times) // 2]
         cpu_baseline = {"value": round(workloads.norm_quant_bytes(rows, H, 1) / t_med / 1e9, 3), "unit": "GB/s",
                         "cores": torch.get_num_threads(), "kind": "port",
-                        "sample": f"restated torch reference (oracle/torch_oracle.py) on CPU tensors, first {rows} of {T} "
+                        "sample": f"restated torch reference (oracle/torch_oracle.py) on CPU tensors, "
+                                  f"{'all' if rows == T else 'first ' + str(rows) + ' of'} {T} "
                                   f"rows x {H}, median of {len(times)} calls over {time.perf_counter() - t_start:.1f} s "
                                   f"({t_med * 1e3:.0f} ms/call); host reports {ncores} cpus"}
 
@@ -273,7 +292,27 @@ def main():
         dst = torch.empty_like(src)
         cp_ms = event_time_ms(lambda i=0: capi.copy_bytes(dst, src, nb), 20)
         extras["copy_kernel_GBps"] = round(2 * nb / (cp_ms * 1e-3) / 1e9, 1)
-        del src, dst
+
+        def copy_same_bytes_us(nbytes):
+            """The plain copy kernel moving as many bytes as a call of a fused kernel moves (half in, half out)."""
+            half = (nbytes // 2 + 15) // 16 * 16
+            room = nb - half
+            offs = [(k * half) % room // 256 * 256 for k in range(3)]   # three windows of the 512 MiB buffers
+            return round(event_time_ms(lambda i=0: capi.copy_bytes(dst[offs[i % 3]:], src[offs[i % 3]:], half), 100) * 1e3, 2)
+
+        # the fused kernel's own memory traffic without its arithmetic (same launch shape, mapping, streaming accesses
+        # and barriers) on the benchmark's buffers: the ceiling of the access pattern, beside the kernel itself
+        def skeleton_step(i=0):
+            x, r, ro, codes, sc = sets[i % NSETS]
+            capi.add_rmsnorm_quant_traffic_only(x, r, ro, codes, sc)
+
+        sk_ms = event_time_ms(skeleton_step, 200)
+        k_ms = event_time_ms(step, 200)
+        extras["add_rmsnorm_quant_traffic_skeleton"] = {
+            "traffic_skeleton_us": round(sk_ms * 1e3, 2), "kernel_us": round(k_ms * 1e3, 2),
+            "kernel_over_skeleton": round(k_ms / sk_ms, 4),
+            "skeleton_frac_of_8TBps": round(alg_bytes / (sk_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "copy_same_bytes_us": copy_same_bytes_us(alg_bytes)}
 
         def rope_case(r, n_sets):
             n_axes = 3 if r.mrope_section is not None else 1
@@ -294,8 +333,8 @@ def main():
                                      r.num_heads_v, r.head_size, r.is_neox, r.eps, q_out, kc, vc, loc, r.k_scale,
                                      r.v_scale, r.mrope_section, r.is_interleaved)
 
+            burst = event_time_ms(call, 200)
             avg, med, mn = per_launch_ms(call, 100)
-            burst = event_time_ms(call, 100)
             return nbytes, avg, med, mn, burst
 
         for name, r in (("rope_kv_qwen3_T4096", workloads.config3()), ("mrope_kv_qwen2vl_T8192", workloads.config4())):
@@ -303,7 +342,9 @@ def main():
             extras[name] = {"us_per_call": round(burst * 1e3, 2), "avg_launch_us": round(avg * 1e3, 2),
                             "GBps": round(nbytes / (burst * 1e-3) / 1e9, 1),
                             "frac_of_8TBps": round(nbytes / (burst * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                            "algorithmic_bytes": nbytes}
+                            "algorithmic_bytes": nbytes, "copy_same_bytes_us": copy_same_bytes_us(nbytes),
+                            "kernel": "rope_rms_walk_kernel (token-walking, one dispatch round of up to 4096 waves)"}
+        del src, dst
 
         # the two-stream op at the reference script's shape (test/test_fused_rope_rms_2way.py:223-246), and the no-KV
         # mRoPE op on the Qwen2-VL-like shape
@@ -345,7 +386,7 @@ def main():
         # 20 distinct buffer sets (GPU-side cost)
         decode = {}
         NG = 20
-        for t in workloads.DECODE_TOKENS:
+        for t in workloads.DECODE_TOKENS_WIDE:
             d = workloads.config5_norm(t)
             g_ = d.gamma.to(dev)
             nq = [(d.x.to(dev).clone(), d.residual.to(dev).clone(), torch.empty((t, 7168), dtype=torch.bfloat16, device=dev),
@@ -368,7 +409,13 @@ def main():
                 capi.rope_rms_set_kv(qkv, qw, kw, cs, pos, t, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
                                      r.is_neox, r.eps, q_out, kc, vc, loc, r.k_scale, r.v_scale)
 
+            def nq_skeleton_call(i=0):
+                x, r_, ro, codes, sc = nq[i % NG]
+                capi.add_rmsnorm_quant_traffic_only(x, r_, ro, codes, sc)
+
             decode[str(t)] = {"add_rmsnorm_quant_us": round(graph_time_us(nq_call, NG), 2),
+                              "add_rmsnorm_quant_traffic_skeleton_us": round(graph_time_us(nq_skeleton_call, NG), 2),
+                              "add_rmsnorm_quant_bytes": workloads.norm_quant_bytes(t, 7168, 1),
                               "rope_kv_fp8_us": round(graph_time_us(rope_call, NG), 2),
                               "add_rmsnorm_quant_eager_us": round(event_time_ms(nq_call, 200) * 1e3, 2),
                               "rope_kv_fp8_eager_us": round(event_time_ms(rope_call, 200) * 1e3, 2)}
@@ -423,7 +470,7 @@ def main():
             del block, cache
 
     out = {
-        "metric": "HBM GB/s add+RMSNorm+FP8 per-token quant @8192x8192 bf16",
+        "metric": f"HBM GB/s add+RMSNorm+FP8 per-token quant @{T}x{H} bf16",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",

@@ -156,14 +156,19 @@ class GPUKDistEnv:
     def allreduce_add_rms_fused(self, allreduce_in, residual_in, rms_weight, eps, fp8_out=False, static_scale=None):
         """gpuk/__init__.py:175-205.  Returns (residual_out, norm_out, scale_out).
 
-        `static_scale` (additive): a 1-element fp32 tensor; selects per-tensor static quantisation.
+        `static_scale` (additive): a 1-element fp32 tensor on the activations' device; selects per-tensor static
+        quantisation.
         """
         self.capture_(allreduce_in)
         residual_out = torch.empty_like(residual_in)
         if fp8_out:
             norm_out = torch.empty_like(allreduce_in, dtype=fp8)
             if static_scale is not None:
-                scale_out = static_scale.reshape(1).to(device=allreduce_in.device, dtype=torch.float32).contiguous()
+                # read by the kernel as it is: a copy or cast made here would be a hidden transfer inside the call,
+                # which a stream capture rejects
+                if static_scale.device != allreduce_in.device or static_scale.dtype != torch.float32 or static_scale.numel() != 1:
+                    raise ValueError("static_scale must be a 1-element fp32 tensor on the device of the activations")
+                scale_out = static_scale.reshape(1)
                 quant = QUANT_FP8_STATIC
             else:
                 scale_out = torch.empty(allreduce_in.shape[0], 1, dtype=torch.float32, device=allreduce_in.device)

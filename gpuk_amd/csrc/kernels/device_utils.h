@@ -47,12 +47,21 @@ template <> struct Pack16<FP16> {
     static __device__ __forceinline__ float hi(uint32_t w) {
         return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
     }
+    // The empty asm statements keep the fp32 value a result of its own: where the compiler sees a product or a
+    // fused multiply-add feeding the conversion it emits v_fma_mixlo_f16, which rounds the exact result once, to
+    // half precision -- not the fp32 rounding followed by the half rounding of the sequence being reproduced
+    // (they differ when the fp32 rounding lands on a half-precision tie).
     static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        asm("" : "+v"(a));
+        asm("" : "+v"(b));
         const uint32_t l = __builtin_bit_cast(uint16_t, (_Float16)a);
         const uint32_t h = __builtin_bit_cast(uint16_t, (_Float16)b);
         return l | (h << 16);
     }
-    static __device__ __forceinline__ float round(float a) { return (float)(_Float16)a; }
+    static __device__ __forceinline__ float round(float a) {
+        asm("" : "+v"(a));
+        return (float)(_Float16)a;
+    }
     static __device__ __forceinline__ float add_squares(uint32_t w, float acc) {
         const float a = lo(w), b = hi(w);
         return __builtin_fmaf(b, b, __builtin_fmaf(a, a, acc));

@@ -17,7 +17,8 @@ from typing import List, Optional
 
 import torch
 
-DECODE_TOKENS = (1, 8, 32, 128, 512)
+DECODE_TOKENS = (1, 8, 32, 128, 512)          # the benchmark definition's decode sweep
+DECODE_TOKENS_WIDE = (1, 8, 32, 128, 256, 512, 1024, 2048)   # the same with the mid-range filled in
 
 
 @dataclass

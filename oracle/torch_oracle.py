@@ -163,17 +163,19 @@ def rope_rms_ref(
     num_tokens: int, num_heads_q: int, num_heads_k: int, num_heads_v: int, head_size: int,
     is_neox_style: bool, eps: float,
     mrope_section: Optional[Sequence[int]] = None, is_interleaved: bool = False,
+    rstd_ulp_offset: int = 0,
 ) -> Tuple[Tensor, Tensor, Tensor]:
     """test/test_fused_rope_rms.py:52-94 (1-D positions) and
     test/test_fused_mrope_rms.py:62-130 (3xT positions).  Returns (q, k, v) as
-    [T, heads, D]; v is the untouched input slice."""
+    [T, heads, D]; v is the untouched input slice.  `rstd_ulp_offset` (test aid, 0 in the
+    reference) moves every head's rstd by that many fp32 ULPs, see rms_norm_forward."""
     q_size = num_heads_q * head_size
     k_size = num_heads_k * head_size
     v_size = num_heads_v * head_size
     qkv = qkv.view(num_tokens, q_size + k_size + v_size)
     q, k, v = qkv.split([q_size, k_size, v_size], dim=-1)
-    q = rms_norm_forward(q.reshape(num_tokens, num_heads_q, head_size), qw, eps)
-    k = rms_norm_forward(k.reshape(num_tokens, num_heads_k, head_size), kw, eps)
+    q = rms_norm_forward(q.reshape(num_tokens, num_heads_q, head_size), qw, eps, rstd_ulp_offset)
+    k = rms_norm_forward(k.reshape(num_tokens, num_heads_k, head_size), kw, eps, rstd_ulp_offset)
     cos, sin = gather_cos_sin(cos_sin, positions, head_size, mrope_section, is_interleaved)
     q = apply_rotary_emb(q, cos, sin, is_neox_style)
     k = apply_rotary_emb(k, cos, sin, is_neox_style)
@@ -187,7 +189,7 @@ def rope_rms_set_kv_ref(
     q_out: Tensor, k_cache: Tensor, v_cache: Tensor, kv_loc: Tensor,
     k_scale: float, v_scale: float,
     mrope_section: Optional[Sequence[int]] = None, is_interleaved: bool = False,
-    scale_same_dtype_cache: bool = False,
+    scale_same_dtype_cache: bool = False, rstd_ulp_offset: int = 0,
 ) -> None:
     """test/test_fused_mrope_rms_set_kv.py:62-130.  Mutates q_out, k_cache, v_cache.
 
@@ -195,7 +197,7 @@ def rope_rms_set_kv_ref(
     float(k)/float(scale) and rounded to bf16, then cast to e4m3fn (:127-128).
     """
     q, k, v = rope_rms_ref(qkv, qw, kw, cos_sin, positions, num_tokens, num_heads_q, num_heads_k,
-                           num_heads_v, head_size, is_neox_style, eps, mrope_section, is_interleaved)
+                           num_heads_v, head_size, is_neox_style, eps, mrope_section, is_interleaved, rstd_ulp_offset)
     if k_cache.dtype != qkv.dtype or scale_same_dtype_cache:
         k = k / k_scale
         v = v / v_scale
@@ -212,15 +214,15 @@ def rope_rms_2way_ref(
     w_q0: Tensor, w_k0: Tensor, w_q1: Tensor, w_k1: Tensor,
     cos_sin0: Tensor, cos_sin1: Tensor,
     batch_size: int, num_tokens0: int, num_tokens1: int, num_heads_q: int, num_heads_k: int,
-    head_size: int, is_interleaved: bool, eps: float,
+    head_size: int, is_interleaved: bool, eps: float, rstd_ulp_offset: int = 0,
 ) -> Tuple[Tensor, Tensor]:
     """test/test_fused_rope_rms_2way.py:37-81: two token streams with their own norm
     weights and per-token cos/sin rows, concatenated along the token axis."""
     is_neox_style = not is_interleaved
-    q0n = rms_norm_forward(q0.view(batch_size, num_tokens0, num_heads_q, head_size), w_q0, eps)
-    k0n = rms_norm_forward(k0.view(batch_size, num_tokens0, num_heads_k, head_size), w_k0, eps)
-    q1n = rms_norm_forward(q1.view(batch_size, num_tokens1, num_heads_q, head_size), w_q1, eps)
-    k1n = rms_norm_forward(k1.view(batch_size, num_tokens1, num_heads_k, head_size), w_k1, eps)
+    q0n = rms_norm_forward(q0.view(batch_size, num_tokens0, num_heads_q, head_size), w_q0, eps, rstd_ulp_offset)
+    k0n = rms_norm_forward(k0.view(batch_size, num_tokens0, num_heads_k, head_size), w_k0, eps, rstd_ulp_offset)
+    q1n = rms_norm_forward(q1.view(batch_size, num_tokens1, num_heads_q, head_size), w_q1, eps, rstd_ulp_offset)
+    k1n = rms_norm_forward(k1.view(batch_size, num_tokens1, num_heads_k, head_size), w_k1, eps, rstd_ulp_offset)
     cos0, sin0 = cos_sin0.view(num_tokens0, head_size).chunk(2, dim=-1)
     cos1, sin1 = cos_sin1.view(num_tokens1, head_size).chunk(2, dim=-1)
     q0o = apply_rotary_emb(q0n, cos0, sin0, is_neox_style)

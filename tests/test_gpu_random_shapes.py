@@ -10,8 +10,7 @@ import torch
 from gpuk_amd import workloads
 from oracle import torch_oracle as O
 from tests.test_gpu_norm_quant import check as check_norm_quant, run_capi as run_norm_quant
-from tests.test_gpu_rope import check_set_kv, oracle_inplace, run_inplace, run_set_kv
-from tests.util import assert_bits_equal, assert_rotated_close
+from tests.test_gpu_rope import check_inplace, check_set_kv, run_inplace, run_set_kv
 
 pytestmark = pytest.mark.gpu
 
@@ -59,8 +58,4 @@ def test_rope_random_shapes(device, tokens, hq, hk, hv, head_size, neox, mrope, 
     inp = make(tokens, hq, head_size, neox, seed=tokens + 100 * hq + hk, mrope=mrope, interleaved=interleaved, fp8=fp8,
                hk=hk, hv=hv)
     check_set_kv(inp, run_set_kv(inp, device), f"[random set_kv {tokens} {hq},{hk},{hv} D={head_size}]")
-    got = run_inplace(inp, device)
-    want = oracle_inplace(inp)
-    nqk = hq + hk
-    assert_rotated_close(got[:, :nqk], want[:, :nqk], "in place q,k")
-    assert_bits_equal(got[:, nqk:], want[:, nqk:], "in place v")
+    check_inplace(inp, run_inplace(inp, device), "in place")

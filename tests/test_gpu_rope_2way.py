@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import c_oracle, torch_oracle as O
-from tests.util import assert_rotated_close
+from tests.util import assert_heads_explained, assert_rotated_close
 
 pytestmark = pytest.mark.gpu
 
@@ -35,11 +35,17 @@ def test_reference_shapes(device, il, B, D):
     T0, T1, Hq, Hk = 678, 3608, 24, 25
     c = make(B, T0, T1, Hq, Hk, D, seed=D + B)
     q01, k01 = run_op(c, B, T0, T1, Hq, Hk, D, il, device)
-    q_ref, k_ref = O.rope_rms_2way_ref(c["q0"], c["k0"], c["q1"], c["k1"], *c["w"], c["cs0"], c["cs1"], B, T0, T1, Hq, Hk,
-                                       D, il, 1e-6)
+    cache = {}
+
+    def want_at(off):
+        if off not in cache:
+            cache[off] = O.rope_rms_2way_ref(c["q0"], c["k0"], c["q1"], c["k1"], *c["w"], c["cs0"], c["cs1"], B, T0, T1,
+                                             Hq, Hk, D, il, 1e-6, off)
+        return cache[off]
+
     assert q01.shape == (B, T0 + T1, Hq, D) and k01.shape == (B, T0 + T1, Hk, D)
-    assert_rotated_close(q01, q_ref, "out_q01")
-    assert_rotated_close(k01, k_ref, "out_k01")
+    assert_heads_explained(q01, lambda off: want_at(off)[0], "out_q01", D)
+    assert_heads_explained(k01, lambda off: want_at(off)[1], "out_k01", D)
 
 
 @pytest.mark.parametrize("B,T0,T1,Hq,Hk,D", [(1, 1, 1, 1, 1, 256), (3, 5, 0, 7, 3, 128), (2, 0, 9, 2, 11, 64),
@@ -68,10 +74,10 @@ def test_fp16_and_rejections(device):
     B, T0, T1, Hq, Hk, D = 2, 6, 4, 3, 2, 128
     c = make(B, T0, T1, Hq, Hk, D, seed=3, dtype=torch.float16)
     q01, k01 = run_op(c, B, T0, T1, Hq, Hk, D, False, device)
-    q_ref, k_ref = O.rope_rms_2way_ref(c["q0"], c["k0"], c["q1"], c["k1"], *c["w"], c["cs0"], c["cs1"], B, T0, T1, Hq, Hk,
-                                       D, False, 1e-6)
-    assert_rotated_close(q01, q_ref, "fp16 q01")
-    assert_rotated_close(k01, k_ref, "fp16 k01")
+    want_at = lambda off: O.rope_rms_2way_ref(c["q0"], c["k0"], c["q1"], c["k1"], *c["w"], c["cs0"], c["cs1"], B, T0, T1, Hq,
+                                              Hk, D, False, 1e-6, off)
+    assert_heads_explained(q01, lambda off: want_at(off)[0], "fp16 q01", D)
+    assert_heads_explained(k01, lambda off: want_at(off)[1], "fp16 k01", D)
     d = lambda t: t.to(device)
     with pytest.raises(RuntimeError):   # token count that does not match the tensors
         gpuk.fused_rope_rms_2way(d(c["q0"]), d(c["k0"]), d(c["q1"]), d(c["k1"]), *[d(w) for w in c["w"]], d(c["cs0"]),
