@@ -55,6 +55,7 @@ struct RopeArgs {
     // token-walking kernel: number of waves in the grid (token stride of a wave) and the token count
     uint32_t walk_waves, num_tokens;
     uint32_t walk_stream;  // 1: q_out / in-place stores (and in-place loads) bypass the L2; for large batches
+    uint32_t walk_merge_rows;  // mRoPE: every aligned group of 8 frequencies takes one axis: rows are merged on load
 };
 
 // dword mask selecting the 16-bit halves whose bit is set in a 2-bit field
@@ -370,6 +371,12 @@ __device__ __forceinline__ void lds_fill16_lanes32(uint32_t lds_byte_offset, con
     asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, %0"
                  : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_offset), "s"(wave_base) : "memory");
 }
+// ... with a full address per lane (the lanes may read from different rows)
+__device__ __forceinline__ void lds_fill16_lanes32_gather(uint32_t lds_byte_offset, const void *lane_address) {
+    uint64_t saved_exec;
+    asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_address) : "memory");
+}
 template <int N>
 __device__ __forceinline__ void wait_fills() {  // until at most N vector memory instructions are outstanding
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -451,10 +458,22 @@ struct RopeWalk {
     float c[8], s[8];      // cos / sin of the current token
     int64_t slot;          // cache slot of the current token
     uint32_t t, u;         // current token and unit
+    int piece_axis;                         // mRoPE: axis of the 16-byte table-row piece this lane fetches
 
     __device__ __forceinline__ RopeWalk(const RopeArgs &args, int lane_)
         : a(args), lane(lane_), sub(lane_ % LPH), hl(lane_ / LPH), heads_qk(args.hq + args.hk),
-          heads_all(args.hq + args.hk + args.hv), v_chunks(SETKV ? args.hv * (D / 8) : 0) {}
+          heads_all(args.hq + args.hk + args.hv), v_chunks(SETKV ? args.hv * (D / 8) : 0) {
+        if constexpr (AXES == 3) {
+            // first frequency of the lane's piece of a table row (cos pieces, then sin pieces); the bitmap words are
+            // picked with selects so that they stay in scalar registers (an index per lane would read them from memory)
+            const uint32_t f = 8 * (((uint32_t)lane % (D / 8)) % (D / 16));
+            auto bit = [&](const uint32_t (&bitmap)[4]) {
+                const uint32_t word = f < 32 ? bitmap[0] : (f < 64 ? bitmap[1] : (f < 96 ? bitmap[2] : bitmap[3]));
+                return (word >> (f & 31)) & 1u;
+            };
+            piece_axis = bit(a.axis2) ? 2 : (bit(a.axis1) ? 1 : 0);
+        }
+    }
 
     __device__ __forceinline__ const uint16_t *token_row(uint32_t tt) const {
         return static_cast<const uint16_t *>(a.qkv_in) + (int64_t)tt * heads_all * D;
@@ -485,6 +504,13 @@ struct RopeWalk {
     // Table row `pos` (2*D bytes: cos | sin) -> 512 bytes at `dst`, repeated 256/D times
     __device__ __forceinline__ void fill_row(uint32_t dst, int64_t pos) const {
         lds_fill16_lanes32(dst, static_cast<const uint16_t *>(a.cos_sin) + pos * D, (16u * lane) % (2u * D));
+    }
+    // mRoPE with every aligned group of 8 frequencies on one axis (chunked sections on multiples of 8): each lane
+    // fetches its 16-byte piece of the row from the table row of that group's axis, so the row arrives merged
+    __device__ __forceinline__ void fill_row_merged(uint32_t dst, int64_t p0, int64_t p1, int64_t p2) const {
+        const uint32_t piece = (uint32_t)lane % (D / 8);  // 16-byte piece of the row: cos pieces, then sin pieces
+        const int64_t pos = piece_axis == 2 ? p2 : (piece_axis == 1 ? p1 : p0);
+        lds_fill16_lanes32_gather(dst, static_cast<const char *>(a.cos_sin) + pos * (2 * D) + 16 * piece);
     }
     // Both weight vectors -> 1 KiB at `dst`: q weights in the first 512 bytes, k weights in the second
     __device__ __forceinline__ void fill_weights(uint32_t dst) const {
@@ -662,6 +688,15 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
     uint32_t mark[RING];  // mark[0]: the current unit, mark[i]: the unit i further on
     bool split = false;   // the three position axes of the token whose rows are staged differ
     auto fill_table = [&](int64_t p0, int64_t p1, int64_t p2) {
+        if constexpr (AXES == 3) {
+            if (a.walk_merge_rows && (p1 != p0 || p2 != p0)) {  // one transfer brings the merged row
+                split = false;
+                w.fill_row_merged(rows_at, p0, p1, p2);
+                issued += 1;
+                rows_mark = issued;
+                return;
+            }
+        }
         w.fill_row(rows_at, p0);
         issued += 1;
         if constexpr (AXES == 3) {
@@ -1033,6 +1068,7 @@ int g_block_threads = 0;    // 0 = default
 int g_walk = 0;             // token-walking kernel: 0 = built-in rule, 1 = never, 2 = always
 int g_walk_waves = 0;       // waves the walking grid may hold at once (0 = built-in)
 int g_walk_stream = 0;      // streaming stores of the walking kernel: 0 = built-in rule, 1 = never, 2 = always
+int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
 
 // Which kernel, measured on MI355X with D = 128 (32/8/8 and 28/4/4 heads, 16-bit cache, random slots):
 //   one wave per unit: best while all units fit the chip about once or twice (decode batches, T = 2048 x 72 heads);
@@ -1163,6 +1199,12 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
         if (section[0] < 0 || section[1] < 0 || section[2] < 0 || section[0] + section[1] + section[2] != D / 2)
             return GPUK_ERR_INVALID_ARG;
         build_axis_bitmaps(section, interleaved != 0, (int)(D / 2), a.axis1, a.axis2);
+        a.walk_merge_rows = 1;
+        for (int f = 0; f < D / 2; f += 8) {
+            const uint32_t g1 = (a.axis1[f >> 5] >> (f & 31)) & 0xffu, g2 = (a.axis2[f >> 5] >> (f & 31)) & 0xffu;
+            if ((g1 != 0 && g1 != 0xffu) || (g2 != 0 && g2 != 0xffu)) a.walk_merge_rows = 0;
+        }
+        if (g_walk_merge_rows == 1) a.walk_merge_rows = 0;
     }
     if (T == 0 || hq + hk + (set_kv ? hv : 0) == 0) return GPUK_OK;
     if (!qkv_in || !qw || !kw || !cos_sin || !positions) return GPUK_ERR_INVALID_ARG;
@@ -1218,6 +1260,7 @@ void set_rope_tuning(int key, int value) {
     if (key == 1) g_walk = value;
     if (key == 2) g_walk_waves = value;
     if (key == 3) g_walk_stream = value;
+    if (key == 4) g_walk_merge_rows = value;
 }
 
 }  // namespace gpuk

@@ -211,7 +211,10 @@ WALK_CASES = [
     (33, (64, 8, 8), 128, False, False, False, True),     # nine units per token, GPT-J pairs, fp8 cache
     (19, (3, 2, 1), 128, True, False, False, False),      # a single, partly filled unit per token
     (23, (7, 2, 0), 128, True, False, False, False),      # no V heads
+    (41, (28, 4, 4), 128, True, "aligned", False, False),  # sections on multiples of 8: the rows arrive merged
+    (27, (6, 2, 2), 64, False, "aligned", False, True),   # the same with GPT-J pairs, head size 64, fp8 cache
 ]
+ALIGNED_SECTIONS = {64: [8, 16, 8], 128: [16, 24, 24], 256: [48, 40, 40]}
 
 
 @pytest.mark.parametrize("case", range(len(WALK_CASES)))
@@ -226,8 +229,11 @@ def test_token_walking_kernel(device, case, waves, stream):
 
     tokens, heads, hs, neox, mrope, interleaved, fp8 = WALK_CASES[case]
     print(f"case walk {WALK_CASES[case]} waves={waves} stream={stream}", flush=True)
-    inp = make(tokens, heads[0], hs, neox, seed=900 + case, mrope=mrope, interleaved=interleaved, fp8=fp8, hk=heads[1],
+    inp = make(tokens, heads[0], hs, neox, seed=900 + case, mrope=bool(mrope), interleaved=interleaved, fp8=fp8, hk=heads[1],
                hv=heads[2])
+    if mrope == "aligned":
+        inp.mrope_section = ALIGNED_SECTIONS[hs]
+        inp.positions[:, ::3] = inp.positions[0, ::3]   # every third token a text token: three equal positions
     if case == 0:   # two padding tokens
         inp.kv_loc[3], inp.kv_loc[tokens - 1] = -1, -5
     nqk = heads[0] + heads[1]
