@@ -460,9 +460,12 @@ struct RopeWalk {
     uint32_t t, u;         // current token and unit
     int piece_axis;                         // mRoPE: axis of the 16-byte table-row piece this lane fetches
 
-    __device__ __forceinline__ RopeWalk(const RopeArgs &args, int lane_)
-        : a(args), lane(lane_), sub(lane_ % LPH), hl(lane_ / LPH), heads_qk(args.hq + args.hk),
-          heads_all(args.hq + args.hk + args.hv), v_chunks(SETKV ? args.hv * (D / 8) : 0) {
+    const void *const qkv_in, *const cos_sin;  // copies of the kernel's leading arguments, see rope_rms_walk_kernel
+
+    __device__ __forceinline__ RopeWalk(const RopeArgs &args, int lane_, const void *qkv_in_, const void *cos_sin_,
+                                        int heads_qk_, int heads_all_, int hv_)
+        : a(args), lane(lane_), sub(lane_ % LPH), hl(lane_ / LPH), heads_qk(heads_qk_), heads_all(heads_all_),
+          v_chunks(SETKV ? hv_ * (D / 8) : 0), qkv_in(qkv_in_), cos_sin(cos_sin_) {
         if constexpr (AXES == 3) {
             // first frequency of the lane's piece of a table row (cos pieces, then sin pieces); the bitmap words are
             // picked with selects so that they stay in scalar registers (an index per lane would read them from memory)
@@ -476,7 +479,7 @@ struct RopeWalk {
     }
 
     __device__ __forceinline__ const uint16_t *token_row(uint32_t tt) const {
-        return static_cast<const uint16_t *>(a.qkv_in) + (int64_t)tt * heads_all * D;
+        return static_cast<const uint16_t *>(qkv_in) + (int64_t)tt * heads_all * D;
     }
     __device__ __forceinline__ bool unit_has_v(uint32_t uu) const { return SETKV && (int)(uu * 64) < v_chunks; }
 
@@ -503,14 +506,14 @@ struct RopeWalk {
     }
     // Table row `pos` (2*D bytes: cos | sin) -> 512 bytes at `dst`, repeated 256/D times
     __device__ __forceinline__ void fill_row(uint32_t dst, int64_t pos) const {
-        lds_fill16_lanes32(dst, static_cast<const uint16_t *>(a.cos_sin) + pos * D, (16u * lane) % (2u * D));
+        lds_fill16_lanes32(dst, static_cast<const uint16_t *>(cos_sin) + pos * D, (16u * lane) % (2u * D));
     }
     // mRoPE with every aligned group of 8 frequencies on one axis (chunked sections on multiples of 8): each lane
     // fetches its 16-byte piece of the row from the table row of that group's axis, so the row arrives merged
     __device__ __forceinline__ void fill_row_merged(uint32_t dst, int64_t p0, int64_t p1, int64_t p2) const {
         const uint32_t piece = (uint32_t)lane % (D / 8);  // 16-byte piece of the row: cos pieces, then sin pieces
         const int64_t pos = piece_axis == 2 ? p2 : (piece_axis == 1 ? p1 : p0);
-        lds_fill16_lanes32_gather(dst, static_cast<const char *>(a.cos_sin) + pos * (2 * D) + 16 * piece);
+        lds_fill16_lanes32_gather(dst, static_cast<const char *>(cos_sin) + pos * (2 * D) + 16 * piece);
     }
     // Both weight vectors -> 1 KiB at `dst`: q weights in the first 512 bytes, k weights in the second
     __device__ __forceinline__ void fill_weights(uint32_t dst) const {
@@ -656,7 +659,12 @@ struct RopeWalk {
 
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 __global__ void __launch_bounds__(kWalkWaves * 64)
-rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__restrict__ kv_loc, const RopeArgs a) {
+rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__restrict__ kv_loc, const void *qkv_in,
+                     const void *cos_sin, uint32_t n_waves, uint32_t tokens, uint32_t upt, int heads_qk, int heads_all,
+                     int ps_token, int ps_axis, int hv, const RopeArgs a) {
+    // The arguments ahead of `a` are what a wave needs to issue its first transfers and the loads of its first
+    // positions.  (Having them preloaded into scalar registers at wave launch, -amdgpu-kernarg-preload-count, was
+    // measured: no difference.)
     using Walk = RopeWalk<T, D, NEOX, AXES, SETKV, KVFP8>;
     constexpr int HPW = Walk::HPW, RING = kWalkRing;
     __shared__ u32x4 s_stage[kWalkWaves][RING][128];  // per wave: the staged units, 2 KiB each
@@ -664,19 +672,18 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
     __shared__ u32x4 s_rows[kWalkWaves][AXES * 32];   // per wave: the table rows of one token, 512 bytes each
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t first = blockIdx.x * kWalkWaves + wave;
-    const uint32_t n_waves = a.walk_waves, tokens = a.num_tokens, upt = a.units_per_token;
-    if (first >= n_waves) return;  // the host keeps walk_waves <= num_tokens
-    Walk w(a, threadIdx.x & 63);
+    if (first >= n_waves) return;  // the host keeps the number of waves <= the number of tokens
+    Walk w(a, threadIdx.x & 63, qkv_in, cos_sin, heads_qk, heads_all, hv);
     w.t = first;
     w.u = 0;
     const uint32_t stage_at = lds_offset_of(&s_stage[wave][0][0]), v_at = lds_offset_of(&s_v[wave][0]),
                    rows_at = lds_offset_of(&s_rows[wave][0]);
 
     auto load_positions = [&](uint32_t tt, int64_t &p0, int64_t &p1, int64_t &p2) {
-        p0 = positions[(int64_t)tt * a.ps_token];
+        p0 = positions[(int64_t)tt * ps_token];
         if constexpr (AXES == 3) {
-            p1 = positions[a.ps_axis + (int64_t)tt * a.ps_token];
-            p2 = positions[2 * a.ps_axis + (int64_t)tt * a.ps_token];
+            p1 = positions[ps_axis + (int64_t)tt * ps_token];
+            p2 = positions[2 * (int64_t)ps_axis + (int64_t)tt * ps_token];
         } else {
             p1 = p2 = p0;
         }
@@ -1085,7 +1092,8 @@ template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 int launch_one(const RopeArgs &a, hipStream_t stream) {
     // the walking kernel shares a token's V row out over the token's units, one 16-byte chunk per lane and unit
     const bool v_fits = !SETKV || (int64_t)a.units_per_token * 64 >= (int64_t)a.hv * (D / 8);
-    const bool walk = v_fits && (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits));
+    const bool strides_fit = a.ps_token == (int)a.ps_token && a.ps_axis == (int)a.ps_axis;  // passed as 32-bit
+    const bool walk = v_fits && strides_fit && (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits));
     if (walk) {
         // every wave the same number of tokens (the last ones one fewer)
         const uint32_t capacity = g_walk_waves ? (uint32_t)g_walk_waves : kWalkCapacity;
@@ -1098,7 +1106,9 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
                                                (KVFP8 ? 1 : 2) * ((int64_t)a.num_tokens * a.hk * D + elems_v)
                                          : 4 * elems_qk;
         b.walk_stream = g_walk_stream == 2 || (g_walk_stream == 0 && walk_bytes >= kWalkStreamBytes) ? 1u : 0u;
-        rope_rms_walk_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<(b.walk_waves + kWalkWaves - 1) / kWalkWaves, kWalkWaves * 64, 0, stream>>>(a.positions, a.kv_loc, b);
+        rope_rms_walk_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<(b.walk_waves + kWalkWaves - 1) / kWalkWaves, kWalkWaves * 64, 0, stream>>>(
+            a.positions, a.kv_loc, a.qkv_in, a.cos_sin, b.walk_waves, a.num_tokens, a.units_per_token, a.hq + a.hk,
+            a.hq + a.hk + a.hv, (int)a.ps_token, (int)a.ps_axis, a.hv, b);
         return hip_status(hipGetLastError());
     }
     const int threads = g_block_threads ? g_block_threads : 256;
@@ -1216,11 +1226,9 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
         if (!aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache)) return GPUK_ERR_MISALIGNED;
         if (kv_fp8 && !(k_scale > 0.f && v_scale > 0.f)) return GPUK_ERR_INVALID_ARG;
     }
-    // one wave per group of 64/(D/16) consecutive Q/K heads of a token; with a KV cache and no Q/K heads at all the
-    // token still gets the waves its V row needs
+    // one wave (or one step of a walking wave) per group of 64/(D/16) consecutive Q/K heads of a token
     const int64_t hpw = 64 / (D / 16);
     int64_t upt = (hq + hk + hpw - 1) / hpw;
-    if (upt == 0) upt = (hv * (D / 8) + 63) / 64;
     if (hq + hk == 0) return GPUK_ERR_UNSUPPORTED;  // a qkv row without Q and K heads has nothing to rotate
     if (dtype == GPUK_DTYPE_F32) upt = hq + hk + (set_kv ? hv : 0);  // the fp32 path: one wave per head
     // mulhi(unit, ceil(2^32/upt)) equals unit / upt while unit * upt < 2^32

@@ -10,6 +10,8 @@ namespace gpuk_ops {
 namespace {
 // amax divisor / clamp bound of the fp8 modes.  448 = OCP e4m3fn (gfx950 hardware); 240 reproduces
 // the reference's fp8e4m3fn::max_value (src/common/float8.h:216-218, gpuk/__init__.py:42-46).
+// One value for the whole process: it changes the numerics of every later allreduce_rms call from any thread (the
+// store itself is atomic).  Set it once at start-up, not around individual calls.
 std::atomic<double> g_fp8_max{448.0};
 }  // namespace
 

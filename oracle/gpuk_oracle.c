@@ -28,9 +28,10 @@
  *   rope: t = rT(a*c), u = rT(b*s), o = rT(t -/+ u)   (three roundings per output)
  *   fp8 KV: code = e4m3fn(rT(f32(k) / scale))
  *
- * Pinned by tests/test_oracle_c.py against torch-CPU library routines (exhaustive
- * e4m3fn table over all bf16 patterns, bf16/fp16 rounding over sampled fp32) and
- * against oracle/torch_oracle.py on seeded inputs.
+ * Pinned by tests/test_oracle_formats.py against torch-CPU library routines (exhaustive
+ * e4m3fn table over all bf16 patterns, bf16/fp16 rounding over sampled fp32) and by
+ * tests/test_oracle_norm_quant.py and tests/test_oracle_rope.py against oracle/torch_oracle.py
+ * on seeded inputs.
  *
  * Deviations from torch semantics, both documented in the header of torch_oracle.py:
  * zero rows give scale 1; a cache of the activation dtype is written unscaled.
