@@ -750,7 +750,7 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
     int64_t slot_next = SETKV ? kv_loc[first] : 0;
     if (first + n_waves < tokens) load_positions(first + n_waves, np0, np1, np2);
     fill_table(p0, p1, p2);
-    wait_fills_upto(issued - weights_mark);
+    wait_fills_upto(__builtin_amdgcn_readfirstlane(issued - weights_mark));
     w.take_weights(reinterpret_cast<const unsigned char *>(&s_v[wave][0]));  // before the V transfer below
     if (w.unit_has_v(0)) {
         w.fill_v(v_at, first, 0);
@@ -767,7 +767,7 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
         uint32_t newest = mark[0];  // the newest transfer this step reads
         if (cur_v) newest = max(newest, v_mark);
         if (token_start) newest = max(newest, rows_mark);
-        wait_fills_upto(issued - newest);
+        wait_fills_upto(__builtin_amdgcn_readfirstlane(issued - newest));  // uniform anyway; keeps the switch scalar
         const u32x4 *stage = &s_stage[wave][0][0] + cslot * 128;
         u32x4 xa = stage[w.lane], xb = stage[64 + w.lane], v = u32x4{0, 0, 0, 0};
         in_registers(xa);
@@ -1077,14 +1077,21 @@ int g_walk_waves = 0;       // waves the walking grid may hold at once (0 = buil
 int g_walk_stream = 0;      // streaming stores of the walking kernel: 0 = built-in rule, 1 = never, 2 = always
 int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
 
-// Which kernel, measured on MI355X with D = 128 (32/8/8 and 28/4/4 heads, 16-bit cache, random slots):
-//   one wave per unit: best while all units fit the chip about once or twice (decode batches, T = 2048 x 72 heads);
-//   token-walking    : from about 20,000 units on; 18.6 against 20.3 us at T = 4096 x 40 heads, 28.1 against 31.2 us at
-//                      T = 8192 x 32 heads;
+// Which kernel, measured on MI355X with D = 128 (32/8/8, 28/4/4 and 64/8/8 heads, random slots):
+//   token-walking    : wins where its waves fill the chip's wave slots: 19.2 against 21.0 us at T = 4096 x 40 heads,
+//                      35.6 against 38.9 at 8192, 51.2 against 60.5 at 12288, 27.5 against 31.5 at 8192 x 32 heads.
+//                      Every wave walks ceil(T / capacity) tokens, so just above a multiple of the capacity few waves
+//                      run (T = 4100: 2050 waves of two tokens) and the other kernel is faster: 23.7 against 21.2 us
+//                      at 4100, 25.5 against 23.3 at 4608, 25.8 against 25.0 at 5120, 42.8 against 37.6 at
+//                      5000 x 72 heads; from two thirds of the slots on the walking kernel is level or ahead (16.4
+//                      against 16.9 at 3072, 28.7 against 28.9 at 6144, 37.1 against 39.2 at 8200);
+//   one wave per unit: everything else: decode batches, and the stretches where the walking grid would be thin;
 //   streaming stores : q_out (or the in-place rows, then with streaming loads too) bypass the L2 once a call moves
 //                      more than the caches absorb: 34.5 against 41.0 us at T = 8192 x 40 heads (203 MB), 69.9 against
 //                      82.5 us at T = 16384, but 19.5 against 18.6 us at T = 4096 (102 MB) and no difference at 153 MB.
-constexpr int64_t kWalkMinUnits = 20000;
+// (Cutting a token's units into runs shared by neighbouring waves, to fill the slots at any T, was measured too: it
+// narrows the dips -- 22.1 us at 4608 -- but never beats the better of the two kernels by more than 5 %.)
+constexpr int64_t kWalkMinUnits = 10000;
 constexpr int64_t kWalkStreamBytes = 176'000'000;
 constexpr uint32_t kWalkCapacity = 4096;  // waves the chip holds at once at 4 per SIMD: one dispatch round
 
@@ -1093,13 +1100,16 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
     // the walking kernel shares a token's V row out over the token's units, one 16-byte chunk per lane and unit
     const bool v_fits = !SETKV || (int64_t)a.units_per_token * 64 >= (int64_t)a.hv * (D / 8);
     const bool strides_fit = a.ps_token == (int)a.ps_token && a.ps_axis == (int)a.ps_axis;  // passed as 32-bit
-    const bool walk = v_fits && strides_fit && (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits));
+    // every wave the same number of tokens (the last ones one fewer)
+    const uint32_t capacity = g_walk_waves ? (uint32_t)g_walk_waves : kWalkCapacity;
+    const uint32_t tokens_per_wave = (a.num_tokens + capacity - 1) / capacity;
+    const uint32_t walk_waves = (a.num_tokens + tokens_per_wave - 1) / tokens_per_wave;
+    const bool slots_filled = 3 * (uint64_t)walk_waves >= 2 * (uint64_t)capacity;
+    const bool walk = v_fits && strides_fit &&
+                      (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits && slots_filled));
     if (walk) {
-        // every wave the same number of tokens (the last ones one fewer)
-        const uint32_t capacity = g_walk_waves ? (uint32_t)g_walk_waves : kWalkCapacity;
-        const uint32_t tokens_per_wave = (a.num_tokens + capacity - 1) / capacity;
         RopeArgs b = a;
-        b.walk_waves = (a.num_tokens + tokens_per_wave - 1) / tokens_per_wave;
+        b.walk_waves = walk_waves;
         // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
         const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
         const int64_t walk_bytes = SETKV ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +

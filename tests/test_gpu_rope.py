@@ -259,10 +259,11 @@ def test_token_walking_kernel(device, case, waves, stream):
 
 
 def test_kernel_choice_by_batch_size(device):
-    """The built-in rule: small batches take the one-wave-per-unit kernel, large ones the walking kernel; with too
-    many V heads for the walking kernel's sharing-out of the V row the first one runs whatever the size.  All of
-    them meet the oracle (sizes on both sides of the switch)."""
-    for tokens, heads in ((3900, (32, 8, 8)), (4100, (32, 8, 8)), (20100, (4, 4, 10))):
+    """The built-in rule: the walking kernel where its waves fill at least two thirds of the chip's wave slots (2731
+    tokens and more; not just above 4096, where every wave would take two tokens and half the slots stay empty), the
+    one-wave-per-unit kernel elsewhere; with too many V heads for the walking kernel's sharing-out of the V row the
+    latter runs whatever the size.  All of them meet the oracle (sizes on both sides of each switch)."""
+    for tokens, heads in ((2700, (32, 8, 8)), (2800, (32, 8, 8)), (4100, (32, 8, 8)), (5800, (12, 4, 4)), (20100, (4, 4, 10))):
         inp = make(tokens, heads[0], 128, True, seed=tokens, hk=heads[1], hv=heads[2])
         check_set_kv(inp, run_set_kv(inp, device), f"[T={tokens} heads={heads}]")
 
