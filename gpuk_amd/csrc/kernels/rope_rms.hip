@@ -1121,7 +1121,11 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
             a.hq + a.hk + a.hv, (int)a.ps_token, (int)a.ps_axis, a.hv, b);
         return hip_status(hipGetLastError());
     }
-    const int threads = g_block_threads ? g_block_threads : 256;
+    // Workgroup size, swept over 64/128/256/512 lanes and one workgroup per token for 2-9 units per token, T = 128-2048:
+    // four waves where a workgroup then holds whole tokens (its waves share the token's position and table row in
+    // the CU's caches: 3-9 % ahead at 28+4 heads), single waves otherwise (2-6 % ahead at 64+8 heads with an fp8 cache,
+    // within 1-3 % either way for 3, 5 and 6 units per token); 128 lanes is the slowest in most cases.
+    const int threads = g_block_threads ? g_block_threads : (a.units_per_token % 4 == 0 ? 256 : 64);
     const uint32_t units_per_block = threads / 64;
     const uint32_t blocks = (a.total_units + units_per_block - 1) / units_per_block;
     rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<blocks, threads, 0, stream>>>(a);
