@@ -246,3 +246,23 @@ def test_reference_kernel_library_exports_its_entry_points():
     # argument refusal happens before any launch
     assert L.gpuk_ref_epilogue_rows(None, None, None, None, None, None, 0, 4096, 1e-6, 1, None) == -1
     assert L.gpuk_ref_rope_rms(None, None, None, None, None, 0, 1, 1, 4, 2, 2, 2, 96, 1, None, 0, 1e-6, None) == -1
+
+
+def test_launch_shape_report():
+    """gpuk_add_rmsnorm_quant_launch_shape computes on the host: lanes per row and 16-byte chunks per lane of the launch
+    the norm-quant entry point would make (no GPU needed)."""
+    from gpuk_amd import capi
+
+    assert capi.add_rmsnorm_quant_launch_shape(8192, 8192) == (512, 2)
+    assert capi.add_rmsnorm_quant_launch_shape(512, 7168) == (448, 2)
+    assert capi.add_rmsnorm_quant_launch_shape(1, 4096) == (256, 2)
+    lanes, chunks = capi.add_rmsnorm_quant_launch_shape(4, 65600 * 2)    # rows that do not stay in registers
+    assert chunks == 0 and lanes % 64 == 0
+    lanes, chunks = capi.add_rmsnorm_quant_launch_shape(128, 1024, torch.float32)
+    assert chunks == 0 and lanes == 256
+    L = capi.lib()
+    import ctypes as C
+    a, b = C.c_int(0), C.c_int(0)
+    assert L.gpuk_add_rmsnorm_quant_launch_shape(0, 1024, 0, C.byref(a), C.byref(b)) == 1
+    assert L.gpuk_add_rmsnorm_quant_launch_shape(4, 1027, 0, C.byref(a), C.byref(b)) == 2
+    assert L.gpuk_add_rmsnorm_quant_launch_shape(4, 1024, 0, None, C.byref(b)) == 1

@@ -404,3 +404,30 @@ def test_static_scale_too_small_saturates(device, fp8_max):
     codes = got[1].cpu().view(torch.uint8) & 0x7F
     top = 0x7E if fp8_max == 448.0 else 0x77
     assert (codes == top).float().mean() > 0.3 and (codes <= top).all()
+
+
+@pytest.mark.parametrize("tokens,hidden", [(5, 1032), (64, 7168), (1030, 8192), (3, 40960)])
+def test_traffic_only_twin_touches_what_the_kernel_touches(device, tokens, hidden):
+    """The calibration entry point moves the norm-quant kernel's bytes without its arithmetic: residual_out = x ^ r
+    bit for bit, one scale of 1.0 per row, codes folded from the same words; nothing beyond the three outputs is
+    written (guard rows before and after each), whatever the launch shape (ragged last wave, the per-XCD row runs
+    of 16 KiB rows, eight chunks per lane)."""
+    from gpuk_amd import capi
+
+    print(f"case traffic-only {tokens}x{hidden}", flush=True)
+    g = torch.Generator().manual_seed(tokens + hidden)
+    x = torch.randint(-2**15, 2**15, (tokens, hidden), generator=g, dtype=torch.int16)
+    r = torch.randint(-2**15, 2**15, (tokens, hidden), generator=g, dtype=torch.int16)
+    res = torch.full((tokens + 2, hidden), 0x5A5A, dtype=torch.int16, device=device)
+    codes = torch.full((tokens + 2, hidden), 0x5A, dtype=torch.uint8, device=device)
+    scale = torch.full((tokens + 2,), -7.0, dtype=torch.float32, device=device)
+    capi.add_rmsnorm_quant_traffic_only(x.to(device).view(torch.bfloat16), r.to(device).view(torch.bfloat16),
+                                        res[1:-1].view(torch.bfloat16), codes[1:-1], scale[1:-1])
+    torch.cuda.synchronize()
+    assert torch.equal(res[1:-1].cpu(), x ^ r)
+    assert (res[0] == 0x5A5A).all() and (res[-1] == 0x5A5A).all()
+    assert (codes[0] == 0x5A).all() and (codes[-1] == 0x5A).all()
+    assert scale[0].item() == -7.0 and scale[-1].item() == -7.0 and (scale[1:-1] == 1.0).all()
+    words = (x ^ r).view(torch.int32).to(torch.int64) & 0xFFFFFFFF          # [tokens, hidden / 2] 32-bit words
+    folded = ((words[:, 0::2] + words[:, 1::2]) & 0xFFFFFFFF).to(torch.int32)  # word 2k + word 2k+1
+    assert torch.equal(codes[1:-1].cpu().view(torch.int32), folded.view(torch.int32))
