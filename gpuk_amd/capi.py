@@ -17,7 +17,7 @@ EXPORTS = ("gpuk_status_string", "gpuk_abi_version", "gpuk_add_rmsnorm_quant", "
            "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_increment_floats", "gpuk_set_tuning",
            "gpuk_add_rmsnorm_quant_traffic_only", "gpuk_add_rmsnorm_quant_launch_shape")
 
-DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2, torch.float64: 3}
 QUANT_NONE, QUANT_FP8_DYNAMIC, QUANT_FP8_E4M3FNUZ, QUANT_FP8_STATIC = 0, 1, 2, 3
 KV_SAME, KV_E4M3FN = 0, 1
 

@@ -322,17 +322,21 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
     }
 }
 
-// fp32 activations: the reference dispatches them through the same template (src/ops/all_reduce_fusion.cpp:375-378).
-// A compatibility path, not a tuned one: three sweeps over the row like the long-row kernel, 4 elements per chunk.
-// Rounding to the activation type is the identity here, so the oracle's sequence is plain fp32 arithmetic:
-// res = x + r; n = gamma * (res * rstd); code = e4m3fn(clamp(n / scale)).
-typedef float f32x4 __attribute__((ext_vector_type(4)));
+// fp32 and fp64 activations: the reference dispatches them through the same template
+// (AT_DISPATCH_FLOATING_TYPES_AND2, src/ops/all_reduce_fusion.cpp:375-378).  A compatibility path, not a tuned one:
+// three sweeps over the row like the long-row kernel, 4 elements per chunk.  Rounding to the activation type is the
+// identity here, so the oracle's sequence is plain arithmetic in that type around an fp32 variance:
+//   res = x + r;  rstd = 1/sqrt(mean(float(res)^2) + eps) in fp32;  n = gamma * (res * F(rstd));
+//   scale = max|float(n)| / fp8_max in fp32;  code = e4m3fn(float(clamp(n / F(scale))))
+// (for F = double torch promotes tensor * fp32-tensor products to double and casts double -> float -> fp8).
+template <typename F>
+using wide4 = F __attribute__((ext_vector_type(4)));
 
-template <int QUANT>
+template <typename F, int QUANT>
 __global__ void __launch_bounds__(kMaxThreads)
-add_rmsnorm_quant_f32_rows(const f32x4 *__restrict__ x, const f32x4 *__restrict__ residual_in,
-                           const f32x4 *__restrict__ gamma, f32x4 *residual_out, void *__restrict__ norm_out,
-                           float *__restrict__ scale_io, int chunks_per_row, float hidden_f, float eps, float fp8_max) {
+add_rmsnorm_quant_wide_rows(const wide4<F> *__restrict__ x, const wide4<F> *__restrict__ residual_in,
+                            const wide4<F> *__restrict__ gamma, wide4<F> *residual_out, void *__restrict__ norm_out,
+                            float *__restrict__ scale_io, int chunks_per_row, float hidden_f, float eps, float fp8_max) {
     __shared__ float s_sum[kReduceSlots];
     __shared__ float s_max[kReduceSlots];
     const int tid = threadIdx.x;
@@ -341,31 +345,34 @@ add_rmsnorm_quant_f32_rows(const f32x4 *__restrict__ x, const f32x4 *__restrict_
 
     float ss = 0.f;
     for (int c = tid; c < chunks_per_row; c += blockDim.x) {
-        const f32x4 res = x[row_base + c] + residual_in[row_base + c];
+        const wide4<F> res = x[row_base + c] + residual_in[row_base + c];
         residual_out[row_base + c] = res;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) ss = __builtin_fmaf(res[j], res[j], ss);
+        for (int j = 0; j < 4; ++j) {
+            const float r = (float)res[j];
+            ss = __builtin_fmaf(r, r, ss);
+        }
     }
     float sumsq[1] = {ss};
     block_allreduce<SumOp, 1>(sumsq, s_sum, num_waves);
-    const float rstd = 1.0f / sqrtf(sumsq[0] / hidden_f + eps);
+    const F rstd = (F)(1.0f / sqrtf(sumsq[0] / hidden_f + eps));
 
     auto normed = [&](int c) {
-        const f32x4 v = residual_out[row_base + c];  // written by this lane above
+        const wide4<F> v = residual_out[row_base + c];  // written by this lane above
         return gamma[c] * (v * rstd);
     };
 
     if constexpr (QUANT == GPUK_QUANT_NONE) {
-        f32x4 *out = reinterpret_cast<f32x4 *>(norm_out) + row_base;
+        wide4<F> *out = reinterpret_cast<wide4<F> *>(norm_out) + row_base;
         for (int c = tid; c < chunks_per_row; c += blockDim.x) out[c] = normed(c);
     } else {
         float scale;
         if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
             float amax = 0.f;
             for (int c = tid; c < chunks_per_row; c += blockDim.x) {
-                const f32x4 v = normed(c);
+                const wide4<F> v = normed(c);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) amax = MaxOp::apply(amax, __builtin_fabsf(v[j]));
+                for (int j = 0; j < 4; ++j) amax = MaxOp::apply(amax, __builtin_fabsf((float)v[j]));
             }
             float am[1] = {amax};
             block_allreduce<MaxOp, 1>(am, s_max, num_waves);
@@ -374,11 +381,13 @@ add_rmsnorm_quant_f32_rows(const f32x4 *__restrict__ x, const f32x4 *__restrict_
         } else {
             scale = scale_io[0];
         }
+        const F wide_scale = (F)scale;
         uint32_t *out = reinterpret_cast<uint32_t *>(norm_out) + row_base;
         for (int c = tid; c < chunks_per_row; c += blockDim.x) {
-            const f32x4 v = normed(c);
-            out[c] = cvt4_e4m3fn(clamp_sym(v[0] / scale, fp8_max), clamp_sym(v[1] / scale, fp8_max),
-                                 clamp_sym(v[2] / scale, fp8_max), clamp_sym(v[3] / scale, fp8_max));
+            const wide4<F> q = normed(c) / wide_scale;
+            // clamping after the cast to fp32 equals the oracle's clamp before it: the bounds are fp32 numbers
+            out[c] = cvt4_e4m3fn(clamp_sym((float)q[0], fp8_max), clamp_sym((float)q[1], fp8_max),
+                                 clamp_sym((float)q[2], fp8_max), clamp_sym((float)q[3], fp8_max));
         }
     }
 }
@@ -455,28 +464,29 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
     return hip_status(hipGetLastError());
 }
 
-template <int QUANT>
-int launch_f32(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
-               float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream) {
+template <typename F, int QUANT>
+int launch_wide(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
+                float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream) {
     const int chunks = (int)(hidden / 4);
     const int want = (chunks + 63) / 64 * 64;
     const int threads = want < kMaxThreads ? want : kMaxThreads;
-    add_rmsnorm_quant_f32_rows<QUANT><<<dim3((unsigned)tokens), threads, 0, stream>>>(
-        static_cast<const f32x4 *>(x), static_cast<const f32x4 *>(residual_in), static_cast<const f32x4 *>(gamma),
-        static_cast<f32x4 *>(residual_out), norm_out, scale, chunks, (float)hidden, eps, fp8_max);
+    add_rmsnorm_quant_wide_rows<F, QUANT><<<dim3((unsigned)tokens), threads, 0, stream>>>(
+        static_cast<const wide4<F> *>(x), static_cast<const wide4<F> *>(residual_in), static_cast<const wide4<F> *>(gamma),
+        static_cast<wide4<F> *>(residual_out), norm_out, scale, chunks, (float)hidden, eps, fp8_max);
     return hip_status(hipGetLastError());
 }
 
-int launch_quant_f32(int quant_mode, const void *x, const void *residual_in, const void *gamma, void *residual_out,
-                     void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max,
-                     hipStream_t stream) {
+template <typename F>
+int launch_quant_wide(int quant_mode, const void *x, const void *residual_in, const void *gamma, void *residual_out,
+                      void *norm_out, float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max,
+                      hipStream_t stream) {
     switch (quant_mode) {
         case GPUK_QUANT_NONE:
-            return launch_f32<GPUK_QUANT_NONE>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+            return launch_wide<F, GPUK_QUANT_NONE>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
         case GPUK_QUANT_FP8_DYNAMIC:
-            return launch_f32<GPUK_QUANT_FP8_DYNAMIC>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+            return launch_wide<F, GPUK_QUANT_FP8_DYNAMIC>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
         case GPUK_QUANT_FP8_STATIC:
-            return launch_f32<GPUK_QUANT_FP8_STATIC>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
+            return launch_wide<F, GPUK_QUANT_FP8_STATIC>(x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, stream);
         default:
             return GPUK_ERR_UNSUPPORTED;
     }
@@ -540,9 +550,10 @@ extern "C" int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidde
                                                    int *chunks_per_lane) {
     using namespace gpuk;
     if (tokens <= 0 || hidden <= 0 || !lanes_per_row || !chunks_per_lane) return GPUK_ERR_INVALID_ARG;
-    const int elems = dtype == GPUK_DTYPE_F32 ? 4 : 8;
+    const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
+    const int elems = wide ? 4 : 8;
     if (hidden % elems != 0) return GPUK_ERR_UNSUPPORTED;
-    if (dtype == GPUK_DTYPE_F32) {  // the fp32 path sweeps the row: lanes only
+    if (wide) {  // the fp32 / fp64 path sweeps the row: lanes only
         const int want = ((int)(hidden / 4) + 63) / 64 * 64;
         *lanes_per_row = want < kMaxThreads ? want : kMaxThreads;
         *chunks_per_lane = 0;
@@ -573,7 +584,9 @@ extern "C" int gpuk_add_rmsnorm_quant(const void *x, const void *residual_in, co
         case GPUK_DTYPE_FP16:
             return launch_quant<FP16>(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
         case GPUK_DTYPE_F32:
-            return launch_quant_f32(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
+            return launch_quant_wide<float>(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
+        case GPUK_DTYPE_F64:
+            return launch_quant_wide<double>(quant_mode, x, residual_in, gamma, residual_out, norm_out, scale, tokens, hidden, eps, fp8_max, s);
         default:
             return GPUK_ERR_UNSUPPORTED;
     }

@@ -823,12 +823,14 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// fp32 activations: the reference dispatches them through the same templates (src/ops/fused_rope.cpp:27-30, :108-111).
-// A compatibility path, not a tuned one: one wave per (token, head), lane l owns rotation pairs l, l+64, ...;
-// with a KV cache the V heads get waves of their own that copy or quantise.  Rounding to the activation type is the
-// identity, so the oracle's sequence is plain fp32 arithmetic with every product rounded before the add.
-template <int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
-__global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
+// fp32 and fp64 activations: the reference dispatches them through the same templates (AT_DISPATCH_FLOATING_TYPES_AND2,
+// src/ops/fused_rope.cpp:27-30, :108-111).  A compatibility path, not a tuned one: one wave per (token, head), lane l
+// owns rotation pairs l, l+64, ...; with a KV cache the V heads get waves of their own that copy or quantise.
+// Rounding to the activation type F is the identity, so the oracle's sequence is plain arithmetic in F with every
+// product rounded before the add, around an fp32 variance and rstd (torch promotes x * rstd to F); an fp8 cache
+// takes float(o / F(scale)).
+template <typename F, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
+__global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
     constexpr int HALF = D / 2;
     constexpr int PPL = (HALF + 63) / 64;  // pairs per lane
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -838,7 +840,7 @@ __global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
     const uint32_t t = a.upt_magic ? __umulhi(unit, a.upt_magic) : unit;
     const int h = (int)(unit - t * a.units_per_token);  // head index inside the token's qkv row
     const int heads_qk = a.hq + a.hk, heads_all = heads_qk + a.hv;
-    const float *src = static_cast<const float *>(a.qkv_in) + ((int64_t)t * heads_all + h) * D;
+    const F *src = static_cast<const F *>(a.qkv_in) + ((int64_t)t * heads_all + h) * D;
 
     if (h >= heads_qk) {  // a V head: only reached with a KV cache
         if constexpr (SETKV) {
@@ -846,12 +848,12 @@ __global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
             if (slot < 0) return;  // token without a cache slot
             const int64_t row = (slot * a.hv + (h - heads_qk)) * D;
             for (int e = lane; e < D; e += 64) {
-                const float v = src[e];
+                const F v = src[e];
                 if constexpr (KVFP8) {
                     static_cast<uint8_t *>(a.v_cache)[row + e] =
-                        (uint8_t)cvt4_e4m3fn(clamp_sym(v / a.v_scale, kE4M3Max), 0.f, 0.f, 0.f);
+                        (uint8_t)cvt4_e4m3fn(clamp_sym((float)(v / (F)a.v_scale), kE4M3Max), 0.f, 0.f, 0.f);
                 } else {
-                    static_cast<float *>(a.v_cache)[row + e] = v;
+                    static_cast<F *>(a.v_cache)[row + e] = v;
                 }
             }
         }
@@ -859,8 +861,8 @@ __global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
     }
 
     const bool is_q = h < a.hq;
-    const float *w = static_cast<const float *>(is_q ? a.qw : a.kw);
-    float x1[PPL], x2[PPL];
+    const F *w = static_cast<const F *>(is_q ? a.qw : a.kw);
+    F x1[PPL], x2[PPL];
     int i1[PPL], i2[PPL];
     bool live[PPL];
     float ss = 0.f;
@@ -871,32 +873,33 @@ __global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
         const int pc = live[k] ? p : 0;
         i1[k] = NEOX ? pc : 2 * pc;
         i2[k] = NEOX ? pc + HALF : 2 * pc + 1;
-        x1[k] = live[k] ? src[i1[k]] : 0.f;
-        x2[k] = live[k] ? src[i2[k]] : 0.f;
-        ss = __builtin_fmaf(x1[k], x1[k], ss);
-        ss = __builtin_fmaf(x2[k], x2[k], ss);
+        x1[k] = live[k] ? src[i1[k]] : (F)0;
+        x2[k] = live[k] ? src[i2[k]] : (F)0;
+        const float f1 = (float)x1[k], f2 = (float)x2[k];
+        ss = __builtin_fmaf(f1, f1, ss);
+        ss = __builtin_fmaf(f2, f2, ss);
     }
     ss = wave_allreduce<SumOp>(ss);
-    const float rstd = 1.0f / sqrtf(ss * (1.0f / D) + a.eps);
+    const F rstd = (F)(1.0f / sqrtf(ss * (1.0f / D) + a.eps));
 
-    const float *table = static_cast<const float *>(a.cos_sin);
+    const F *table = static_cast<const F *>(a.cos_sin);
     const int64_t p0 = a.positions[(int64_t)t * a.ps_token];
     int64_t p1 = p0, p2 = p0;
     if constexpr (AXES == 3) {
         p1 = a.positions[a.ps_axis + (int64_t)t * a.ps_token];
         p2 = a.positions[2 * a.ps_axis + (int64_t)t * a.ps_token];
     }
-    float *dst;
+    F *dst;
     uint8_t *dst8 = nullptr;
     if constexpr (!SETKV) {
-        dst = static_cast<float *>(a.qkv_out) + ((int64_t)t * heads_all + h) * D;
+        dst = static_cast<F *>(a.qkv_out) + ((int64_t)t * heads_all + h) * D;
     } else if (is_q) {
-        dst = static_cast<float *>(a.q_out) + ((int64_t)t * a.hq + h) * D;
+        dst = static_cast<F *>(a.q_out) + ((int64_t)t * a.hq + h) * D;
     } else {
         const int64_t slot = a.kv_loc[t];
         if (slot < 0) return;  // token without a cache slot: nothing of a K head is kept
         const int64_t row = (slot * a.hk + (h - a.hq)) * D;
-        dst = static_cast<float *>(a.k_cache) + row;          // used when the cache is fp32
+        dst = static_cast<F *>(a.k_cache) + row;              // used when the cache has the activation type
         dst8 = static_cast<uint8_t *>(a.k_cache) + row;       // used when it is fp8
     }
 #pragma unroll
@@ -908,12 +911,12 @@ __global__ void __launch_bounds__(256) rope_rms_f32_kernel(const RopeArgs a) {
             const bool on1 = (a.axis1[f >> 5] >> (f & 31)) & 1u, on2 = (a.axis2[f >> 5] >> (f & 31)) & 1u;
             pos = on2 ? p2 : (on1 ? p1 : p0);
         }
-        const float c = table[pos * D + f], s = table[pos * D + HALF + f];
-        const float n1 = w[i1[k]] * (x1[k] * rstd), n2 = w[i2[k]] * (x2[k] * rstd);
-        const float o1 = n1 * c - n2 * s, o2 = n2 * c + n1 * s;
+        const F c = table[pos * D + f], s = table[pos * D + HALF + f];
+        const F n1 = w[i1[k]] * (x1[k] * rstd), n2 = w[i2[k]] * (x2[k] * rstd);
+        const F o1 = n1 * c - n2 * s, o2 = n2 * c + n1 * s;
         if (SETKV && KVFP8 && !is_q) {
-            dst8[i1[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym(o1 / a.k_scale, kE4M3Max), 0.f, 0.f, 0.f);
-            dst8[i2[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym(o2 / a.k_scale, kE4M3Max), 0.f, 0.f, 0.f);
+            dst8[i1[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym((float)(o1 / (F)a.k_scale), kE4M3Max), 0.f, 0.f, 0.f);
+            dst8[i2[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym((float)(o2 / (F)a.k_scale), kE4M3Max), 0.f, 0.f, 0.f);
         } else {
             dst[i1[k]] = o1;
             dst[i2[k]] = o2;
@@ -982,11 +985,12 @@ __global__ void __launch_bounds__(256) rope_rms_2way_kernel(const TwoWayArgs a) 
     }
 }
 
-// fp32 form of the two-stream op (the reference dispatches float here too: src/ops/fused_rope.cpp:197-200): one wave
-// per (token, head) row of a segment, lane l owns rotation pairs l, l+64, ...; plain fp32 arithmetic, every product
-// rounded before the add.  The host counts one unit per row for this kernel.
-template <int D, bool NEOX>
-__global__ void __launch_bounds__(256) rope_rms_2way_f32_kernel(const TwoWayArgs a) {
+// fp32 / fp64 form of the two-stream op (the reference dispatches float and double here too:
+// src/ops/fused_rope.cpp:197-200): one wave per (token, head) row of a segment, lane l owns rotation pairs l, l+64, ...;
+// plain arithmetic in the activation type F around an fp32 variance, every product rounded before the add.  The host
+// counts one unit per row for this kernel.
+template <typename F, int D, bool NEOX>
+__global__ void __launch_bounds__(256) rope_rms_2way_wide_kernel(const TwoWayArgs a) {
     constexpr int HALF = D / 2;
     constexpr int PPL = (HALF + 63) / 64;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1001,13 +1005,13 @@ __global__ void __launch_bounds__(256) rope_rms_2way_f32_kernel(const TwoWayArgs
     const uint32_t token = a.heads_magic[kind] ? __umulhi(row, a.heads_magic[kind]) : row;
     const uint32_t head = row - token * heads;
 
-    const float *src = static_cast<const float *>(a.in[seg]) + ((int64_t)batch * rows + row) * D;
-    const float *w = static_cast<const float *>(a.w[seg]);
-    const float *table = static_cast<const float *>(a.cos_sin[stream_id]) + (int64_t)token * D;
+    const F *src = static_cast<const F *>(a.in[seg]) + ((int64_t)batch * rows + row) * D;
+    const F *w = static_cast<const F *>(a.w[seg]);
+    const F *table = static_cast<const F *>(a.cos_sin[stream_id]) + (int64_t)token * D;
     const int64_t out_token = (int64_t)batch * (a.tokens0 + a.tokens1) + (stream_id ? a.tokens0 : 0) + token;
-    float *dst = static_cast<float *>(a.out[kind]) + (out_token * heads + head) * D;
+    F *dst = static_cast<F *>(a.out[kind]) + (out_token * heads + head) * D;
 
-    float x1[PPL], x2[PPL];
+    F x1[PPL], x2[PPL];
     int i1[PPL], i2[PPL];
     bool live[PPL];
     float ss = 0.f;
@@ -1018,19 +1022,20 @@ __global__ void __launch_bounds__(256) rope_rms_2way_f32_kernel(const TwoWayArgs
         const int pc = live[k] ? p : 0;
         i1[k] = NEOX ? pc : 2 * pc;
         i2[k] = NEOX ? pc + HALF : 2 * pc + 1;
-        x1[k] = live[k] ? src[i1[k]] : 0.f;
-        x2[k] = live[k] ? src[i2[k]] : 0.f;
-        ss = __builtin_fmaf(x1[k], x1[k], ss);
-        ss = __builtin_fmaf(x2[k], x2[k], ss);
+        x1[k] = live[k] ? src[i1[k]] : (F)0;
+        x2[k] = live[k] ? src[i2[k]] : (F)0;
+        const float f1 = (float)x1[k], f2 = (float)x2[k];
+        ss = __builtin_fmaf(f1, f1, ss);
+        ss = __builtin_fmaf(f2, f2, ss);
     }
     ss = wave_allreduce<SumOp>(ss);
-    const float rstd = 1.0f / sqrtf(ss * (1.0f / D) + a.eps);
+    const F rstd = (F)(1.0f / sqrtf(ss * (1.0f / D) + a.eps));
 #pragma unroll
     for (int k = 0; k < PPL; ++k) {
         if (!live[k]) continue;
         const int f = lane + 64 * k;
-        const float c = table[f], s = table[HALF + f];
-        const float n1 = w[i1[k]] * (x1[k] * rstd), n2 = w[i2[k]] * (x2[k] * rstd);
+        const F c = table[f], s = table[HALF + f];
+        const F n1 = w[i1[k]] * (x1[k] * rstd), n2 = w[i2[k]] * (x2[k] * rstd);
         dst[i1[k]] = n1 * c - n2 * s;
         dst[i2[k]] = n2 * c + n1 * s;
     }
@@ -1044,19 +1049,20 @@ int launch_2way(const TwoWayArgs &a, bool neox, unsigned batch, hipStream_t stre
     return hip_status(hipGetLastError());
 }
 
-template <int D>
-int launch_2way_f32(const TwoWayArgs &a, bool neox, unsigned batch, hipStream_t stream) {
+template <typename F, int D>
+int launch_2way_wide(const TwoWayArgs &a, bool neox, unsigned batch, hipStream_t stream) {
     const dim3 grid((a.unit_end[3] + 3) / 4, batch);
-    if (neox) rope_rms_2way_f32_kernel<D, true><<<grid, 256, 0, stream>>>(a);
-    else rope_rms_2way_f32_kernel<D, false><<<grid, 256, 0, stream>>>(a);
+    if (neox) rope_rms_2way_wide_kernel<F, D, true><<<grid, 256, 0, stream>>>(a);
+    else rope_rms_2way_wide_kernel<F, D, false><<<grid, 256, 0, stream>>>(a);
     return hip_status(hipGetLastError());
 }
 
-int launch_2way_f32_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned batch, hipStream_t stream) {
+template <typename F>
+int launch_2way_wide_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned batch, hipStream_t stream) {
     switch (D) {
-        case 64: return launch_2way_f32<64>(a, neox, batch, stream);
-        case 128: return launch_2way_f32<128>(a, neox, batch, stream);
-        case 256: return launch_2way_f32<256>(a, neox, batch, stream);
+        case 64: return launch_2way_wide<F, 64>(a, neox, batch, stream);
+        case 128: return launch_2way_wide<F, 128>(a, neox, batch, stream);
+        case 256: return launch_2way_wide<F, 256>(a, neox, batch, stream);
         default: return GPUK_ERR_UNSUPPORTED;
     }
 }
@@ -1151,31 +1157,32 @@ int launch_style(const RopeArgs &a, bool neox, int n_axes, bool set_kv, bool kv_
                        : launch_mode<T, D, false, 1>(a, set_kv, kv_fp8, stream);
 }
 
-template <int D, bool NEOX, int AXES>
-int launch_f32_mode(const RopeArgs &a, bool set_kv, bool kv_fp8, hipStream_t stream) {
+template <typename F, int D, bool NEOX, int AXES>
+int launch_wide_mode(const RopeArgs &a, bool set_kv, bool kv_fp8, hipStream_t stream) {
     const uint32_t blocks = (a.total_units + 3) / 4;
-    if (!set_kv) rope_rms_f32_kernel<D, NEOX, AXES, false, false><<<blocks, 256, 0, stream>>>(a);
-    else if (kv_fp8) rope_rms_f32_kernel<D, NEOX, AXES, true, true><<<blocks, 256, 0, stream>>>(a);
-    else rope_rms_f32_kernel<D, NEOX, AXES, true, false><<<blocks, 256, 0, stream>>>(a);
+    if (!set_kv) rope_rms_wide_kernel<F, D, NEOX, AXES, false, false><<<blocks, 256, 0, stream>>>(a);
+    else if (kv_fp8) rope_rms_wide_kernel<F, D, NEOX, AXES, true, true><<<blocks, 256, 0, stream>>>(a);
+    else rope_rms_wide_kernel<F, D, NEOX, AXES, true, false><<<blocks, 256, 0, stream>>>(a);
     return hip_status(hipGetLastError());
 }
 
-template <int D>
-int launch_f32_style(const RopeArgs &a, bool neox, int n_axes, bool set_kv, bool kv_fp8, hipStream_t stream) {
+template <typename F, int D>
+int launch_wide_style(const RopeArgs &a, bool neox, int n_axes, bool set_kv, bool kv_fp8, hipStream_t stream) {
     if (neox) {
-        return n_axes == 3 ? launch_f32_mode<D, true, 3>(a, set_kv, kv_fp8, stream)
-                           : launch_f32_mode<D, true, 1>(a, set_kv, kv_fp8, stream);
+        return n_axes == 3 ? launch_wide_mode<F, D, true, 3>(a, set_kv, kv_fp8, stream)
+                           : launch_wide_mode<F, D, true, 1>(a, set_kv, kv_fp8, stream);
     }
-    return n_axes == 3 ? launch_f32_mode<D, false, 3>(a, set_kv, kv_fp8, stream)
-                       : launch_f32_mode<D, false, 1>(a, set_kv, kv_fp8, stream);
+    return n_axes == 3 ? launch_wide_mode<F, D, false, 3>(a, set_kv, kv_fp8, stream)
+                       : launch_wide_mode<F, D, false, 1>(a, set_kv, kv_fp8, stream);
 }
 
-int launch_f32_head_size(const RopeArgs &a, int64_t head_size, bool neox, int n_axes, bool set_kv, bool kv_fp8,
-                         hipStream_t stream) {
+template <typename F>
+int launch_wide_head_size(const RopeArgs &a, int64_t head_size, bool neox, int n_axes, bool set_kv, bool kv_fp8,
+                          hipStream_t stream) {
     switch (head_size) {
-        case 64: return launch_f32_style<64>(a, neox, n_axes, set_kv, kv_fp8, stream);
-        case 128: return launch_f32_style<128>(a, neox, n_axes, set_kv, kv_fp8, stream);
-        case 256: return launch_f32_style<256>(a, neox, n_axes, set_kv, kv_fp8, stream);
+        case 64: return launch_wide_style<F, 64>(a, neox, n_axes, set_kv, kv_fp8, stream);
+        case 128: return launch_wide_style<F, 128>(a, neox, n_axes, set_kv, kv_fp8, stream);
+        case 256: return launch_wide_style<F, 256>(a, neox, n_axes, set_kv, kv_fp8, stream);
         default: return GPUK_ERR_UNSUPPORTED;
     }
 }
@@ -1216,7 +1223,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     if (T < 0 || hq < 0 || hk < 0 || hv < 0) return GPUK_ERR_INVALID_ARG;
     if (n_axes != 1 && n_axes != 3) return GPUK_ERR_INVALID_ARG;
     if (D != 64 && D != 128 && D != 256) return GPUK_ERR_UNSUPPORTED;
-    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32) return GPUK_ERR_UNSUPPORTED;
+    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32 && dtype != GPUK_DTYPE_F64) return GPUK_ERR_UNSUPPORTED;
     if (set_kv && kv_dtype != GPUK_KV_SAME && kv_dtype != GPUK_KV_E4M3FN) return GPUK_ERR_UNSUPPORTED;
     if (hq > 0x7fffff || hk > 0x7fffff || hv > 0x7fffff) return GPUK_ERR_UNSUPPORTED;
     RopeArgs a{};
@@ -1246,7 +1253,8 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     const int64_t hpw = 64 / (D / 16);
     int64_t upt = (hq + hk + hpw - 1) / hpw;
     if (hq + hk == 0) return GPUK_ERR_UNSUPPORTED;  // a qkv row without Q and K heads has nothing to rotate
-    if (dtype == GPUK_DTYPE_F32) upt = hq + hk + (set_kv ? hv : 0);  // the fp32 path: one wave per head
+    const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
+    if (wide) upt = hq + hk + (set_kv ? hv : 0);  // the fp32 / fp64 path: one wave per head
     // mulhi(unit, ceil(2^32/upt)) equals unit / upt while unit * upt < 2^32
     if (upt * T >= 0x7fffffffLL || upt * T * upt >= (1LL << 32)) return GPUK_ERR_UNSUPPORTED;
     a.qkv_in = qkv_in;
@@ -1272,7 +1280,8 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     a.k_scale = k_scale;
     a.v_scale = v_scale;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == GPUK_DTYPE_F32) return launch_f32_head_size(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
+    if (dtype == GPUK_DTYPE_F32) return launch_wide_head_size<float>(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
+    if (dtype == GPUK_DTYPE_F64) return launch_wide_head_size<double>(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
     if (dtype == GPUK_DTYPE_BF16) return launch_head_size<BF16>(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
     return launch_head_size<FP16>(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
 }
@@ -1321,9 +1330,10 @@ extern "C" int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1
     using namespace gpuk;
     if (batch_size < 0 || num_tokens0 < 0 || num_tokens1 < 0 || num_heads_q < 0 || num_heads_k < 0) return GPUK_ERR_INVALID_ARG;
     if (head_size != 64 && head_size != 128 && head_size != 256) return GPUK_ERR_UNSUPPORTED;
-    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32) return GPUK_ERR_UNSUPPORTED;
+    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32 && dtype != GPUK_DTYPE_F64) return GPUK_ERR_UNSUPPORTED;
     if (batch_size > 65535) return GPUK_ERR_UNSUPPORTED;  // grid.y
-    const int64_t hpw = dtype == GPUK_DTYPE_F32 ? 1 : 64 / (head_size / 16);  // rows (heads) per wave
+    const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
+    const int64_t hpw = wide ? 1 : 64 / (head_size / 16);  // rows (heads) per wave
     const int64_t rows[4] = {num_tokens0 * num_heads_q, num_tokens0 * num_heads_k, num_tokens1 * num_heads_q,
                              num_tokens1 * num_heads_k};
     const void *ins[4] = {q0, k0, q1, k1};
@@ -1361,7 +1371,8 @@ extern "C" int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1
     a.eps = eps;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool neox = !is_interleaved;  // reference: fused_rope.cpp:168-227 dispatches the NeoX kernel when !is_interleaved
-    if (dtype == GPUK_DTYPE_F32) return launch_2way_f32_head_size(a, head_size, neox, (unsigned)batch_size, s);
+    if (dtype == GPUK_DTYPE_F32) return launch_2way_wide_head_size<float>(a, head_size, neox, (unsigned)batch_size, s);
+    if (dtype == GPUK_DTYPE_F64) return launch_2way_wide_head_size<double>(a, head_size, neox, (unsigned)batch_size, s);
     if (dtype == GPUK_DTYPE_BF16) return launch_2way_head_size<BF16>(a, head_size, neox, (unsigned)batch_size, s);
     return launch_2way_head_size<FP16>(a, head_size, neox, (unsigned)batch_size, s);
 }

@@ -30,7 +30,8 @@ inline int activation_dtype(const Tensor &t, const char *op) {
         case at::kBFloat16: return GPUK_DTYPE_BF16;
         case at::kHalf: return GPUK_DTYPE_FP16;
         case at::kFloat: return GPUK_DTYPE_F32;
-        default: TORCH_CHECK(false, op, ": activations must be bfloat16, float16 or float32, got ", t.scalar_type());
+        case at::kDouble: return GPUK_DTYPE_F64;
+        default: TORCH_CHECK(false, op, ": activations must be bfloat16, float16, float32 or float64, got ", t.scalar_type());
     }
 }
 

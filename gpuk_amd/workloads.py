@@ -71,9 +71,9 @@ class RopeInputs:
             # finite codes only (avoid 0x7f / 0xff NaN patterns so equality checks are plain)
             k = torch.randint(0, 0x7E, shape_k, generator=g, dtype=torch.uint8).view(torch.float8_e4m3fn)
             v = torch.randint(0, 0x7E, shape_v, generator=g, dtype=torch.uint8).view(torch.float8_e4m3fn)
-        elif self.kv_dtype == torch.float32:
-            k = torch.randn(shape_k, generator=g) * 1000.0
-            v = torch.randn(shape_v, generator=g) * 1000.0
+        elif self.kv_dtype in (torch.float32, torch.float64):
+            k = (torch.randn(shape_k, generator=g) * 1000.0).to(self.kv_dtype)
+            v = (torch.randn(shape_v, generator=g) * 1000.0).to(self.kv_dtype)
         else:
             k = torch.randint(-30000, 30000, shape_k, generator=g, dtype=torch.int16).view(self.kv_dtype)
             v = torch.randint(-30000, 30000, shape_v, generator=g, dtype=torch.int16).view(self.kv_dtype)

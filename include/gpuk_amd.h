@@ -36,7 +36,8 @@ typedef enum gpuk_status {
 typedef enum gpuk_dtype {
     GPUK_DTYPE_BF16 = 0,
     GPUK_DTYPE_FP16 = 1,
-    GPUK_DTYPE_F32 = 2 /* compatibility path (the reference dispatches float too); not tuned like the 16-bit types */
+    GPUK_DTYPE_F32 = 2, /* compatibility paths (the reference dispatches float and double too: */
+    GPUK_DTYPE_F64 = 3  /* AT_DISPATCH_FLOATING_TYPES_AND2); not tuned like the 16-bit types */
 } gpuk_dtype;
 
 /* quant_type of the allreduce_rms op.  0/1/2 are the reference's QuantType
