@@ -357,19 +357,28 @@ __global__ void __launch_bounds__(512) rope_rms_kernel(const RopeArgs a) {
 constexpr int kWalkWaves = 4;  // waves per workgroup of the walking kernel
 constexpr int kWalkRing = 2;   // staging buffers per wave = units in flight beyond the current one
 
+// The base of a transfer has to sit in a pair of scalar registers.  It is wave-uniform by construction; reading it
+// through the first lane makes that hold for the compiler too, whatever it concluded about the loads the address was
+// computed from (for a value it already keeps in scalar registers the reads fold away).  "vcc" is named as clobbered
+// only to keep the allocator from handing it over as that operand, which the instruction does not take.
+__device__ __forceinline__ const void *in_scalar_registers(const void *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo);
+}
 template <bool NT>
 __device__ __forceinline__ void lds_fill16(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
     if constexpr (NT) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(wave_base) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc");
     } else {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(wave_base) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc");
     }
 }
 // the same for lanes 0-31 only: 512 bytes of LDS
 __device__ __forceinline__ void lds_fill16_lanes32(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
     uint64_t saved_exec;
     asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_offset), "s"(wave_base) : "memory");
+                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc");
 }
 // ... with a full address per lane (the lanes may read from different rows)
 __device__ __forceinline__ void lds_fill16_lanes32_gather(uint32_t lds_byte_offset, const void *lane_address) {
