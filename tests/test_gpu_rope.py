@@ -437,3 +437,52 @@ def test_negative_slots_and_colliding_slots(device, fp8):
     rtol = 0.13 if fp8 else 1e-2
     k_close = ((cand_k - got_k[None]).abs() <= 5e-2 + rtol * cand_k.abs()).all(dim=-1).any(dim=0)
     assert bool(k_close.all()), f"K pieces not from any colliding token: {(~k_close).nonzero().flatten().tolist()}"
+
+
+def test_walking_kernel_replayed_from_a_graph(device):
+    """The token-walking kernel (asynchronous global-to-LDS transfers, hand-counted waits) recorded into a HIP graph:
+    every replay, with fresh inputs copied into the captured buffers and eager work in between, equals the eager
+    call on the same inputs."""
+    import gpuk_amd as gpuk
+    from gpuk_amd import capi
+
+    T, hq, hk, hv, D = 300, 28, 4, 4, 128
+    inp = make(T, hq, D, True, seed=71, mrope=True, hk=hk, hv=hv)
+    inp.mrope_section = ALIGNED_SECTIONS[D]
+    qkv, qw, kw, cs, pos, loc = to_dev(inp, device)
+    k0, v0 = inp.new_cache()
+    static_qkv, static_pos = torch.zeros_like(qkv), pos.clone()
+    q_out = torch.empty((T, hq, D), dtype=qkv.dtype, device=device)
+    kc, vc = k0.to(device), v0.to(device)
+
+    def call(src, positions, q, k, v):
+        gpuk.fused_mrope_3d_rms_set_kv(src, qw, kw, cs, positions, T, hq, hk, hv, D, True, inp.mrope_section, False,
+                                       inp.eps, q, k, v, loc, 1.0, 1.0)
+
+    capi.set_tuning("rope_walk", 2)
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            call(static_qkv, static_pos, q_out, kc, vc)    # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            call(static_qkv, static_pos, q_out, kc, vc)
+        for rep in range(4):
+            g = torch.Generator(device=device).manual_seed(200 + rep)
+            x = torch.randn(qkv.shape, device=device, generator=g).to(qkv.dtype)
+            p = torch.randint(0, 10000, (3, T), device=device, generator=g, dtype=torch.int64)
+            p[:, ::4] = p[0, ::4]                           # every fourth token a text token
+            static_qkv.copy_(x)
+            static_pos.copy_(p)
+            graph.replay()
+            torch.cuda.synchronize()
+            q2, k2, v2 = torch.empty_like(q_out), k0.to(device), v0.to(device)
+            call(x, p, q2, k2, v2)
+            torch.cuda.synchronize()
+            raw = lambda t: t.view(torch.int16)
+            assert torch.equal(raw(q_out), raw(q2)), f"replay {rep}: q_out"
+            assert torch.equal(raw(kc[loc]), raw(k2[loc])) and torch.equal(raw(vc[loc]), raw(v2[loc])), f"replay {rep}: cache rows"
+    finally:
+        capi.set_tuning("rope_walk", 0)
