@@ -31,7 +31,7 @@ typedef enum gpuk_status {
     GPUK_ERR_INTERNAL = 5
 } gpuk_status;
 
-/* 16-bit activation formats (the reference dispatches on at::ScalarType:
+/* Activation formats (the reference dispatches on at::ScalarType:
  * src/ops/all_reduce_fusion.cpp:375, src/ops/fused_rope.cpp:27-31). */
 typedef enum gpuk_dtype {
     GPUK_DTYPE_BF16 = 0,
