@@ -677,7 +677,8 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
     using Walk = RopeWalk<T, D, NEOX, AXES, SETKV, KVFP8>;
     constexpr int HPW = Walk::HPW, RING = kWalkRing;
     __shared__ u32x4 s_stage[kWalkWaves][RING][128];  // per wave: the staged units, 2 KiB each
-    __shared__ u32x4 s_v[kWalkWaves][64];             // per wave: one unit's V chunks (first the norm weights)
+    __shared__ u32x4 s_v[kWalkWaves][64];             // per wave: one unit's V chunks
+    __shared__ u32x4 s_w[kWalkWaves][64];             // per wave: the norm weights, read once
     __shared__ u32x4 s_rows[kWalkWaves][AXES * 32];   // per wave: the table rows of one token, 512 bytes each
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t first = blockIdx.x * kWalkWaves + wave;
@@ -686,7 +687,7 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
     w.t = first;
     w.u = 0;
     const uint32_t stage_at = lds_offset_of(&s_stage[wave][0][0]), v_at = lds_offset_of(&s_v[wave][0]),
-                   rows_at = lds_offset_of(&s_rows[wave][0]);
+                   rows_at = lds_offset_of(&s_rows[wave][0]), weights_at = lds_offset_of(&s_w[wave][0]);
 
     auto load_positions = [&](uint32_t tt, int64_t &p0, int64_t &p1, int64_t &p2) {
         p0 = positions[(int64_t)tt * ps_token];
@@ -744,28 +745,36 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
         fslot = fslot + 1 == (uint32_t)RING ? 0 : fslot + 1;
     };
 
-    // prologue.  The weights go first (they arrive soonest and are waited for first), then the first RING units,
-    // then what depends on the first token's positions.
-    w.fill_weights(v_at);
-    issued += 1;
-    const uint32_t weights_mark = issued;
-#pragma unroll
-    for (int i = 0; i < RING; ++i) mark[i] = 0;
-#pragma unroll
-    for (int i = 0; i < RING; ++i) stage_next();
-    // after the transfers above: a wait for these scalar loads placed ahead of them would hold them back
+    // prologue.  The loads of the first positions are issued first and waited for only after the transfers that do
+    // not need them (weights, the first unit, its V share) are on their way; the first token's table row follows,
+    // ahead of the remaining staged units: memory operations complete in issue order, so the first unit can start as
+    // soon as its own data and the row are there, not after everything staged behind them.
+    {   // every kernel argument the transfers below take is in registers before the position loads are issued: a
+        // wait for an argument fetched later would also wait for the positions (scalar loads return in any order,
+        // so the only wait there is waits for all of them)
+        const void *qw_ = a.qw, *kw_ = a.kw;
+        asm volatile("" ::"s"(qkv_in), "s"(cos_sin), "s"(qw_), "s"(kw_), "s"(tokens), "s"(upt), "s"(heads_qk), "s"(heads_all), "s"(hv));
+    }
     int64_t p0, p1, p2, np0 = 0, np1 = 0, np2 = 0;
     load_positions(first, p0, p1, p2);
     int64_t slot_next = SETKV ? kv_loc[first] : 0;
     if (first + n_waves < tokens) load_positions(first + n_waves, np0, np1, np2);
-    fill_table(p0, p1, p2);
-    wait_fills_upto(__builtin_amdgcn_readfirstlane(issued - weights_mark));
-    w.take_weights(reinterpret_cast<const unsigned char *>(&s_v[wave][0]));  // before the V transfer below
+    w.fill_weights(weights_at);
+    issued += 1;
+    const uint32_t weights_mark = issued;
+#pragma unroll
+    for (int i = 0; i < RING; ++i) mark[i] = 0;
+    stage_next();
     if (w.unit_has_v(0)) {
         w.fill_v(v_at, first, 0);
         issued += 1;
         v_mark = issued;
     }
+    fill_table(p0, p1, p2);
+#pragma unroll
+    for (int i = 1; i < RING; ++i) stage_next();
+    wait_fills_upto(__builtin_amdgcn_readfirstlane(issued - weights_mark));
+    w.take_weights(reinterpret_cast<const unsigned char *>(&s_w[wave][0]));
 
     // One step: wait for the current unit's transfers (and, at a token's first unit, for its table rows), move it to
     // registers, refill what that freed (next token's rows, next unit's V share, the unit RING ahead), finish the unit.
