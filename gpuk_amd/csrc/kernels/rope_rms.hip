@@ -1102,14 +1102,19 @@ int g_walk_stream = 0;      // streaming stores of the walking kernel: 0 = built
 int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
 
 // Which kernel, measured on MI355X with D = 128 (32/8/8, 28/4/4 and 64/8/8 heads, random slots):
-//   token-walking    : wins where its waves fill the chip's wave slots: 19.2 against 21.0 us at T = 4096 x 40 heads,
-//                      35.6 against 38.9 at 8192, 51.2 against 60.5 at 12288, 27.5 against 31.5 at 8192 x 32 heads.
-//                      Every wave walks ceil(T / capacity) tokens, so just above a multiple of the capacity few waves
-//                      run (T = 4100: 2050 waves of two tokens) and the other kernel is faster: 23.7 against 21.2 us
-//                      at 4100, 25.5 against 23.3 at 4608, 25.8 against 25.0 at 5120, 42.8 against 37.6 at
-//                      5000 x 72 heads; from two thirds of the slots on the walking kernel is level or ahead (16.4
-//                      against 16.9 at 3072, 28.7 against 28.9 at 6144, 37.1 against 39.2 at 8200);
-//   one wave per unit: everything else: decode batches, and the stretches where the walking grid would be thin;
+//   token-walking    : every wave walks ceil(T / capacity) tokens, and the grid's waves are dealt evenly to the
+//                      chip's 1024 SIMDs, so its run time moves in steps of ceil(waves / 1024) waves per SIMD (one
+//                      token per wave, 40 heads: 9.2 us at 1024 tokens, 12.1 at 2048, 15.4 at 3072, 19.0 at 4096,
+//                      and 14.5-14.8 anywhere from 2400 to 2800) while the other kernel's grows with the tokens
+//                      (7.3 / 12.2 / 17.1 / 21.0 us).  It wins where the last step is nearly full: 14.7 against 15.7 us
+//                      at 2700 tokens, 19.0 against 21.0 at 4096, 35.3 against 38.9 at 8192, 51.2 against 60.5 at
+//                      12288, 27.5 against 31.5 at 8192 x 32 heads, 19.9 against 21.5 at 2048 x 40 heads of 256 -- and
+//                      loses where it is not: 14.5 against 14.1 at 2400, 23.7 against 21.2 at 4100 (2050 waves of two
+//                      tokens), 25.5 against 23.3 at 4608, 22.4 against 20.6 at 2400 x 72 heads; with a single wave
+//                      per SIMD it always loses (9.2 against 7.3 us at 1024 tokens).  With an fp8 cache it is ahead
+//                      only on a full grid (40 heads: 19.8 against 21.3 us at 4096 tokens, but 13.3 against 12.6 at
+//                      2048, 16.0 against 15.7 at 2700, 25.7 against 25.2 at 5300, 32.4 against 31.3 at 7000);
+//   one wave per unit: everything else: decode batches, and the stretches where the walking grid's last step is thin;
 //   streaming stores : q_out (or the in-place rows, then with streaming loads too) bypass the L2 once a call moves
 //                      more than the caches absorb: 34.5 against 41.0 us at T = 8192 x 40 heads (203 MB), 69.9 against
 //                      82.5 us at T = 16384, but 19.5 against 18.6 us at T = 4096 (102 MB) and no difference at 153 MB.
@@ -1118,6 +1123,7 @@ int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allo
 constexpr int64_t kWalkMinUnits = 10000;
 constexpr int64_t kWalkStreamBytes = 176'000'000;
 constexpr uint32_t kWalkCapacity = 4096;  // waves the chip holds at once at 4 per SIMD: one dispatch round
+constexpr uint32_t kComputeUnits = 256;   // MI355X
 
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 int launch_one(const RopeArgs &a, hipStream_t stream) {
@@ -1128,9 +1134,12 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
     const uint32_t capacity = g_walk_waves ? (uint32_t)g_walk_waves : kWalkCapacity;
     const uint32_t tokens_per_wave = (a.num_tokens + capacity - 1) / capacity;
     const uint32_t walk_waves = (a.num_tokens + tokens_per_wave - 1) / tokens_per_wave;
-    // ... or fewer waves of one long token each (head size 256: 19.9 against 21.5 us at T = 2048 x 40 heads)
-    const bool slots_filled = 3 * (uint64_t)walk_waves >= 2 * (uint64_t)capacity ||
-                              (tokens_per_wave == 1 && (int64_t)a.total_units >= 2 * kWalkMinUnits);
+    const uint32_t simds = 4 * kComputeUnits;
+    const uint32_t waves_per_simd = (walk_waves + simds - 1) / simds;  // of the fullest SIMD
+    // with an fp8 cache the other kernel is closer (its stores are half the size, the quantising arithmetic weighs
+    // more in a walking wave): there the walking kernel is ahead only with all four waves per SIMD in place
+    const bool slots_filled = KVFP8 ? 100 * (uint64_t)walk_waves >= 95 * (uint64_t)capacity
+                                    : waves_per_simd >= 2 && 100 * (uint64_t)walk_waves >= 85 * (uint64_t)waves_per_simd * simds;
     const bool walk = v_fits && strides_fit &&
                       (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits && slots_filled));
     if (walk) {

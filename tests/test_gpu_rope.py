@@ -259,13 +259,16 @@ def test_token_walking_kernel(device, case, waves, stream):
 
 
 def test_kernel_choice_by_batch_size(device):
-    """The built-in rule: the walking kernel where its waves fill at least two thirds of the chip's wave slots (2731
-    tokens and more; not just above 4096, where every wave would take two tokens and half the slots stay empty), the
-    one-wave-per-unit kernel elsewhere; with too many V heads for the walking kernel's sharing-out of the V row the
-    latter runs whatever the size.  All of them meet the oracle (sizes on both sides of each switch)."""
-    for tokens, heads in ((2700, (32, 8, 8)), (2800, (32, 8, 8)), (4100, (32, 8, 8)), (5800, (12, 4, 4)), (20100, (4, 4, 10))):
-        inp = make(tokens, heads[0], 128, True, seed=tokens, hk=heads[1], hv=heads[2])
-        check_set_kv(inp, run_set_kv(inp, device), f"[T={tokens} heads={heads}]")
+    """The built-in rule: the walking kernel where the fullest SIMD's share of its waves is matched on nearly all
+    SIMDs (2048 tokens: two waves each; 2700: most of three; not 2400, not just above 4096, where every wave would
+    take two tokens and half the slots stay empty; with an fp8 cache only on a full grid), the one-wave-per-unit
+    kernel elsewhere; with too many V heads for the walking kernel's sharing-out of the V row the latter runs whatever
+    the size.  All of them meet the oracle (sizes on both sides of each switch)."""
+    for tokens, heads, fp8 in ((2048, (32, 8, 8), False), (2400, (32, 8, 8), False), (2700, (32, 8, 8), False),
+                               (4100, (32, 8, 8), False), (5800, (12, 4, 4), False), (3800, (12, 4, 4), True),
+                               (4000, (12, 4, 4), True), (20100, (4, 4, 10), False)):
+        inp = make(tokens, heads[0], 128, True, seed=tokens, fp8=fp8, hk=heads[1], hv=heads[2])
+        check_set_kv(inp, run_set_kv(inp, device), f"[T={tokens} heads={heads} fp8={fp8}]")
 
 
 @pytest.mark.parametrize("hq,hk,hv,head_size", [(3, 1, 40, 64), (1, 1, 17, 256), (7, 2, 0, 128), (2, 9, 33, 128)])
