@@ -167,6 +167,18 @@ __device__ __forceinline__ void norm_rotate(const u32x4 &xa, const u32x4 &xb, co
     }
 }
 
+// A pair of 16-byte stores OFFSET bytes apart, streamed past the L2 (nt) or left to it.  The streaming form is
+// written in assembly: as two arms of a run-time choice, the compiler merges a non-temporal and a plain store into
+// one plain store.
+template <int OFFSET>
+__device__ __forceinline__ void store_pair(void *p, const u32x4 &a, const u32x4 &b, bool nt) {
+    if (nt) {
+        asm volatile("global_store_dwordx4 %0, %1, off nt\n\tglobal_store_dwordx4 %0, %2, off offset:%3 nt" ::"v"(p), "v"(a), "v"(b), "n"(OFFSET) : "memory");
+    } else {
+        *reinterpret_cast<u32x4 *>(p) = a;
+        *reinterpret_cast<u32x4 *>(static_cast<char *>(p) + OFFSET) = b;
+    }
+}
 // What one wave keeps about one unit (= one group of 64/(D/16) consecutive Q/K heads of one token, plus its share
 // of the token's V row) between issuing the unit's loads and finishing it.
 struct UnitState {
@@ -279,8 +291,7 @@ struct RopeUnit {
         if (st.active && (st.is_q || slot_ok)) {
             if constexpr (!SETKV) {
                 uint16_t *dst = static_cast<uint16_t *>(a.qkv_out) + ((int64_t)st.t * heads_all + head) * D;
-                *reinterpret_cast<u32x4 *>(dst + c0(sub)) = oa;
-                *reinterpret_cast<u32x4 *>(dst + c1(sub)) = ob;
+                store_pair<HALF * 2>(dst + c0(sub), oa, ob, a.walk_stream != 0);
             } else if (KVFP8 && !st.is_q) {
                 uint8_t *dst = static_cast<uint8_t *>(a.k_cache) + (st.slot * a.hk + (head - a.hq)) * D;
                 const float s = a.k_scale, rcp = 1.0f / s;
@@ -295,8 +306,7 @@ struct RopeUnit {
                 // q_out row or (16-bit) K cache row of the slot: one store sequence, destination chosen per lane
                 uint16_t *dst = st.is_q ? static_cast<uint16_t *>(a.q_out) + ((int64_t)st.t * a.hq + head) * D
                                         : static_cast<uint16_t *>(a.k_cache) + (st.slot * a.hk + (head - a.hq)) * D;
-                *reinterpret_cast<u32x4 *>(dst + c0(sub)) = oa;
-                *reinterpret_cast<u32x4 *>(dst + c1(sub)) = ob;
+                store_pair<HALF * 2>(dst + c0(sub), oa, ob, a.walk_stream != 0);
             }
         }
 
@@ -407,18 +417,6 @@ __device__ __forceinline__ void wait_fills_upto(uint32_t n) {
 __device__ __forceinline__ void in_registers(u32x4 &v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ uint32_t lds_offset_of(const void *shared_ptr) { return (uint32_t)(uintptr_t)shared_ptr; }
 
-// A pair of 16-byte stores OFFSET bytes apart, streamed past the L2 (nt) or left to it.  The streaming form is
-// written in assembly: as two arms of a run-time choice, the compiler merges a non-temporal and a plain store into
-// one plain store.
-template <int OFFSET>
-__device__ __forceinline__ void store_pair(void *p, const u32x4 &a, const u32x4 &b, bool nt) {
-    if (nt) {
-        asm volatile("global_store_dwordx4 %0, %1, off nt\n\tglobal_store_dwordx4 %0, %2, off offset:%3 nt" ::"v"(p), "v"(a), "v"(b), "n"(OFFSET) : "memory");
-    } else {
-        *reinterpret_cast<u32x4 *>(p) = a;
-        *reinterpret_cast<u32x4 *>(static_cast<char *>(p) + OFFSET) = b;
-    }
-}
 // Same arithmetic as norm_rotate with the weights and the cos/sin values already unpacked to fp32.
 //   w[2j], w[2j+1]     : low / high half of dword j of the first chunk's weights;  w[8+2j], w[8+2j+1]: second chunk
 //   c[e], s[e]         : the lane's 8 cos / sin values in load_trig order
@@ -960,6 +958,7 @@ struct TwoWayArgs {
     uint32_t heads_magic[2];  // ceil(2^32 / heads), 0 for heads == 1
     int tokens0, tokens1;
     float eps;
+    uint32_t stream;  // 1: the output rows are stored past the L2 (calls that move more than a few MB)
 };
 
 template <typename T, int D, bool NEOX>
@@ -998,8 +997,7 @@ __global__ void __launch_bounds__(256) rope_rms_2way_kernel(const TwoWayArgs a) 
     if (active) {
         const int64_t out_token = (int64_t)batch * (a.tokens0 + a.tokens1) + (stream_id ? a.tokens0 : 0) + token;
         uint16_t *dst = static_cast<uint16_t *>(a.out[kind]) + (out_token * heads + head) * D;
-        *reinterpret_cast<u32x4 *>(dst + c0) = oa;
-        *reinterpret_cast<u32x4 *>(dst + c1) = ob;
+        store_pair<HALF * 2>(dst + c0, oa, ob, a.stream != 0);
     }
 }
 
@@ -1101,27 +1099,34 @@ int g_walk_waves = 0;       // waves the walking grid may hold at once (0 = buil
 int g_walk_stream = 0;      // streaming stores of the walking kernel: 0 = built-in rule, 1 = never, 2 = always
 int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
 
-// Which kernel, measured on MI355X with D = 128 (32/8/8, 28/4/4 and 64/8/8 heads, random slots):
+// Which kernel and which stores, measured on MI355X (32/8/8, 28/4/4 and 64/8/8 heads, head sizes 64-256, random slots):
+//   streaming stores : in the one-wave-per-unit kernel, q_out / K rows / in-place rows written past the L2 are ahead
+//                      from about 10 MB per call on (64+8 heads, fp8 cache: 5.9 against 7.0 us at 512 tokens, 16.0
+//                      against 18.1 at 2048; 40 heads: 19.0 against 21.1 us at 4096 tokens, 65.2 against 80.2 at
+//                      16384; level at 5 MB and below) -- what a kernel leaves dirty in the L2 is written back at its
+//                      end.  The walking kernel keeps its rows in the L2 up to 130 MB per call (18.5 against 19.1 us
+//                      at 4096 x 40 heads) and streams them (in place: loads too) above (27.5 against 27.9 us at
+//                      8192 x 32 heads, 35.1 against 41.2 at 8192 x 40);
 //   token-walking    : every wave walks ceil(T / capacity) tokens, and the grid's waves are dealt evenly to the
 //                      chip's 1024 SIMDs, so its run time moves in steps of ceil(waves / 1024) waves per SIMD (one
 //                      token per wave, 40 heads: 9.2 us at 1024 tokens, 12.1 at 2048, 15.4 at 3072, 19.0 at 4096,
-//                      and 14.5-14.8 anywhere from 2400 to 2800) while the other kernel's grows with the tokens
-//                      (7.3 / 12.2 / 17.1 / 21.0 us).  It wins where the last step is nearly full: 14.7 against 15.7 us
-//                      at 2700 tokens, 19.0 against 21.0 at 4096, 35.3 against 38.9 at 8192, 51.2 against 60.5 at
-//                      12288, 27.5 against 31.5 at 8192 x 32 heads, 19.9 against 21.5 at 2048 x 40 heads of 256 -- and
-//                      loses where it is not: 14.5 against 14.1 at 2400, 23.7 against 21.2 at 4100 (2050 waves of two
-//                      tokens), 25.5 against 23.3 at 4608, 22.4 against 20.6 at 2400 x 72 heads; with a single wave
-//                      per SIMD it always loses (9.2 against 7.3 us at 1024 tokens).  With an fp8 cache it is ahead
-//                      only on a full grid (40 heads: 19.8 against 21.3 us at 4096 tokens, but 13.3 against 12.6 at
-//                      2048, 16.0 against 15.7 at 2700, 25.7 against 25.2 at 5300, 32.4 against 31.3 at 7000);
-//   one wave per unit: everything else: decode batches, and the stretches where the walking grid's last step is thin;
-//   streaming stores : q_out (or the in-place rows, then with streaming loads too) bypass the L2 once a call moves
-//                      more than the caches absorb: 34.5 against 41.0 us at T = 8192 x 40 heads (203 MB), 69.9 against
-//                      82.5 us at T = 16384, but 19.5 against 18.6 us at T = 4096 (102 MB) and no difference at 153 MB.
+//                      and 14.5-14.8 anywhere from 2400 to 2800) while the other kernel's grows with the tokens.
+//                      Against the other kernel with streaming stores it is ahead where its last step is full and
+//                      three or four waves sit on every SIMD, and then only (a) with three position axes, where a
+//                      token's merged table row is fetched once instead of three rows per group of heads (28+4
+//                      heads: 16.3 against 17.5 us at 4096 tokens, 21.5 against 24.1 at 6144, 28.0 against 30.2 at
+//                      8192, 52.1 against 54.8 at 16384; 3-4 % with an fp8 cache), and (b) with one axis, a 16-bit
+//                      cache and one token per wave (40 heads of 128: 18.45 against 18.9 us at 4096 tokens, 14.9
+//                      against 15.1 at 3072).  Elsewhere the other kernel is level or ahead: 33.9 against 35.1 us at
+//                      8192 x 40 heads, 65.1 against 68.6 at 16384, 28.0 against 31.5 at 4096 x 72 heads with an fp8
+//                      cache, 65.6 against 70.7 at 8192 x 40 heads of 256, and by 10 % where the walking grid's last
+//                      step is thin (19.2 against 22.8 us at 4100 tokens);
+//   one wave per unit: everything else.
 // (Cutting a token's units into runs shared by neighbouring waves, to fill the slots at any T, was measured too: it
-// narrows the dips -- 22.1 us at 4608 -- but never beats the better of the two kernels by more than 5 %.)
+// narrows the walking kernel's dips -- 22.1 us at 4608 -- but never beats the better of the two kernels.)
 constexpr int64_t kWalkMinUnits = 10000;
-constexpr int64_t kWalkStreamBytes = 176'000'000;
+constexpr int64_t kWalkStreamBytes = 130'000'000;
+constexpr int64_t kUnitStreamBytes = 8'000'000;
 constexpr uint32_t kWalkCapacity = 4096;  // waves the chip holds at once at 4 per SIMD: one dispatch round
 constexpr uint32_t kComputeUnits = 256;   // MI355X
 
@@ -1136,34 +1141,34 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
     const uint32_t walk_waves = (a.num_tokens + tokens_per_wave - 1) / tokens_per_wave;
     const uint32_t simds = 4 * kComputeUnits;
     const uint32_t waves_per_simd = (walk_waves + simds - 1) / simds;  // of the fullest SIMD
-    // with an fp8 cache the other kernel is closer (its stores are half the size, the quantising arithmetic weighs
-    // more in a walking wave): there the walking kernel is ahead only with all four waves per SIMD in place
-    const bool slots_filled = KVFP8 ? 100 * (uint64_t)walk_waves >= 95 * (uint64_t)capacity
-                                    : waves_per_simd >= 2 && 100 * (uint64_t)walk_waves >= 85 * (uint64_t)waves_per_simd * simds;
+    const bool last_step_full = waves_per_simd >= 3 && 100 * (uint64_t)walk_waves >= 95 * (uint64_t)waves_per_simd * simds;
+    const bool slots_filled = last_step_full && (AXES == 3 || (!KVFP8 && D == 128 && tokens_per_wave == 1));
     const bool walk = v_fits && strides_fit &&
                       (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits && slots_filled));
+    RopeArgs b = a;
+    // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
+    const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
+    const int64_t call_bytes = SETKV ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
+                                           (KVFP8 ? 1 : 2) * ((int64_t)a.num_tokens * a.hk * D + elems_v)
+                                     : 4 * elems_qk;
+    const int64_t stream_from = walk ? kWalkStreamBytes : kUnitStreamBytes;
+    b.walk_stream = g_walk_stream == 2 || (g_walk_stream == 0 && call_bytes >= stream_from) ? 1u : 0u;
     if (walk) {
-        RopeArgs b = a;
         b.walk_waves = walk_waves;
-        // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
-        const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
-        const int64_t walk_bytes = SETKV ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
-                                               (KVFP8 ? 1 : 2) * ((int64_t)a.num_tokens * a.hk * D + elems_v)
-                                         : 4 * elems_qk;
-        b.walk_stream = g_walk_stream == 2 || (g_walk_stream == 0 && walk_bytes >= kWalkStreamBytes) ? 1u : 0u;
         rope_rms_walk_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<(b.walk_waves + kWalkWaves - 1) / kWalkWaves, kWalkWaves * 64, 0, stream>>>(
             a.positions, a.kv_loc, a.qkv_in, a.cos_sin, b.walk_waves, a.num_tokens, a.units_per_token, a.hq + a.hk,
             a.hq + a.hk + a.hv, (int)a.ps_token, (int)a.ps_axis, a.hv, b);
         return hip_status(hipGetLastError());
     }
-    // Workgroup size, swept over 64/128/256/512 lanes and one workgroup per token for 2-9 units per token, T = 128-2048:
-    // four waves where a workgroup then holds whole tokens (its waves share the token's position and table row in
-    // the CU's caches: 3-9 % ahead at 28+4 heads), single waves otherwise (2-6 % ahead at 64+8 heads with an fp8 cache,
-    // within 1-3 % either way for 3, 5 and 6 units per token); 128 lanes is the slowest in most cases.
-    const int threads = g_block_threads ? g_block_threads : (a.units_per_token % 4 == 0 ? 256 : 64);
+    // Workgroup size, swept over 64/128/256/512 lanes and one workgroup per token for 2-9 units per token: four waves
+    // where a workgroup then holds whole tokens (its waves share the token's position and table row in the CU's
+    // caches: 3-15 % ahead at 28+4 heads) and for large batches (1-3 % ahead from 4096 tokens on), single waves for
+    // small batches of other head counts (2-6 % ahead at 64+8 heads with an fp8 cache up to 512 tokens, within 1-3 %
+    // either way for 3, 5 and 6 units per token); 128 lanes is the slowest in most cases.
+    const int threads = g_block_threads ? g_block_threads : (a.units_per_token % 4 == 0 || a.total_units > 8192 ? 256 : 64);
     const uint32_t units_per_block = threads / 64;
     const uint32_t blocks = (a.total_units + units_per_block - 1) / units_per_block;
-    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<blocks, threads, 0, stream>>>(a);
+    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<blocks, threads, 0, stream>>>(b);
     return hip_status(hipGetLastError());
 }
 
@@ -1396,6 +1401,10 @@ extern "C" int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1
     a.tokens0 = (int)num_tokens0;
     a.tokens1 = (int)num_tokens1;
     a.eps = eps;
+    {   // as in the one-wave-per-unit rope kernel: streamed stores are ahead from about 10 MB per call on
+        const int64_t call_bytes = 4 * batch_size * (num_tokens0 + num_tokens1) * (num_heads_q + num_heads_k) * head_size;
+        a.stream = g_walk_stream == 2 || (g_walk_stream == 0 && call_bytes >= kUnitStreamBytes) ? 1u : 0u;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool neox = !is_interleaved;  // reference: fused_rope.cpp:168-227 dispatches the NeoX kernel when !is_interleaved
     if (dtype == GPUK_DTYPE_F32) return launch_2way_wide_head_size<float>(a, head_size, neox, (unsigned)batch_size, s);

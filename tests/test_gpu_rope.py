@@ -259,16 +259,18 @@ def test_token_walking_kernel(device, case, waves, stream):
 
 
 def test_kernel_choice_by_batch_size(device):
-    """The built-in rule: the walking kernel where the fullest SIMD's share of its waves is matched on nearly all
-    SIMDs (2048 tokens: two waves each; 2700: most of three; not 2400, not just above 4096, where every wave would
-    take two tokens and half the slots stay empty; with an fp8 cache only on a full grid), the one-wave-per-unit
-    kernel elsewhere; with too many V heads for the walking kernel's sharing-out of the V row the latter runs whatever
-    the size.  All of them meet the oracle (sizes on both sides of each switch)."""
-    for tokens, heads, fp8 in ((2048, (32, 8, 8), False), (2400, (32, 8, 8), False), (2700, (32, 8, 8), False),
-                               (4100, (32, 8, 8), False), (5800, (12, 4, 4), False), (3800, (12, 4, 4), True),
-                               (4000, (12, 4, 4), True), (20100, (4, 4, 10), False)):
-        inp = make(tokens, heads[0], 128, True, seed=tokens, fp8=fp8, hk=heads[1], hv=heads[2])
-        check_set_kv(inp, run_set_kv(inp, device), f"[T={tokens} heads={heads} fp8={fp8}]")
+    """The built-in rule: the walking kernel where three or four of its waves sit on nearly every SIMD (2920-3072 and
+    3892-4096 tokens with one token per wave; the same bands of tokens / tokens per wave above), and then only with
+    three position axes or, with one axis, a 16-bit cache and one token per wave; the one-wave-per-unit kernel
+    elsewhere, with its q_out / K rows streamed past the L2 from 8 MB per call on.  All of them meet the oracle (sizes
+    on both sides of each switch; mRoPE and plain RoPE; an fp8 cache; too many V heads for the walking kernel)."""
+    cases = ((2900, (32, 8, 8), False, False), (3000, (32, 8, 8), False, False), (4100, (32, 8, 8), False, False),
+             (6100, (12, 4, 4), False, True), (5800, (12, 4, 4), False, True), (4000, (12, 4, 4), True, False),
+             (4000, (12, 4, 4), True, True), (300, (32, 8, 8), False, False), (20100, (4, 4, 10), False, False))
+    for tokens, heads, fp8, mrope in cases:
+        inp = make(tokens, heads[0], 128, True, seed=tokens, mrope=mrope, fp8=fp8, hk=heads[1], hv=heads[2])
+        check_set_kv(inp, run_set_kv(inp, device), f"[T={tokens} heads={heads} fp8={fp8} mrope={mrope}]")
+        check_inplace(inp, run_inplace(inp, device), f"[in place T={tokens} heads={heads} mrope={mrope}]")
 
 
 @pytest.mark.parametrize("hq,hk,hv,head_size", [(3, 1, 40, 64), (1, 1, 17, 256), (7, 2, 0, 128), (2, 9, 33, 128)])
