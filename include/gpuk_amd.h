@@ -188,7 +188,7 @@ int gpuk_increment_floats(float *data, int64_t n, void *stream);
  * the built-in choice.  Keys: "norm_quant_nchunk" (1/2/4/8 16-byte chunks per lane), "norm_quant_threads" (lanes
  * per row), "norm_quant_row_group_shift" (log2 of the run of consecutive rows one XCD takes; -1, not 0, restores the
  * built-in rule), "rope_block_threads" (64/128/256/512, one-wave-per-unit kernel), "rope_walk" (token-walking kernel:
- * 1 never, 2 always), "rope_walk_waves" (waves of its grid), "rope_walk_stream" (its streaming stores: 1 never,
+ * 1 never, 2 always), "rope_walk_waves" (waves of its grid), "rope_walk_stream" (output rows of all three rope kernels stored past the L2: 1 never,
  * 2 always), "rope_walk_merge_rows" (1: never fetch an mRoPE token's cos/sin row with one per-lane-addressed
  * transfer).  Unknown keys or values return GPUK_ERR_INVALID_ARG.  The settings are process-global plain variables
  * read at launch: set them from one thread while no other thread is launching.  Not part of the reference. */
