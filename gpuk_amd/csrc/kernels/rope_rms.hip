@@ -253,6 +253,27 @@ struct RopeUnit {
         const int sub = lane % LPH;
         const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin);
         const int64_t p0 = st.p0;
+        if constexpr (AXES == 3) {
+            const int64_t p1 = st.p1, p2 = st.p2;
+            if (a.walk_merge_rows && (p1 != p0 || p2 != p0)) {
+                // every aligned group of 8 frequencies takes one axis: each lane reads its pieces from that axis's row
+                const uint32_t b1 = trig_bits<D, NEOX>(a.axis1, sub), b2 = trig_bits<D, NEOX>(a.axis2, sub);
+                const int64_t pa = (b2 & 1u) ? p2 : ((b1 & 1u) ? p1 : p0);
+                if constexpr (NEOX) {
+                    st.cosv = load_trig<D, NEOX>(table + pa * D, sub);
+                    st.sinv = load_trig<D, NEOX>(table + pa * D + HALF, sub);
+                } else {
+                    const int64_t pb = (b2 & 16u) ? p2 : ((b1 & 16u) ? p1 : p0);
+                    const u32x2 cl = *reinterpret_cast<const u32x2 *>(table + pa * D + 4 * sub);
+                    const u32x2 ch = *reinterpret_cast<const u32x2 *>(table + pb * D + D / 4 + 4 * sub);
+                    const u32x2 sl = *reinterpret_cast<const u32x2 *>(table + pa * D + HALF + 4 * sub);
+                    const u32x2 sh = *reinterpret_cast<const u32x2 *>(table + pb * D + HALF + D / 4 + 4 * sub);
+                    st.cosv = u32x4{cl[0], cl[1], ch[0], ch[1]};
+                    st.sinv = u32x4{sl[0], sl[1], sh[0], sh[1]};
+                }
+                return;
+            }
+        }
         st.cosv = load_trig<D, NEOX>(table + p0 * D, sub);
         st.sinv = load_trig<D, NEOX>(table + p0 * D + HALF, sub);
         if constexpr (AXES == 3) {
