@@ -86,14 +86,31 @@ __device__ __forceinline__ u32x4 load_trig(const uint16_t *row, int sub) {  // r
     }
 }
 // ... and the matching 8 bits of a frequency bitmap (bit f = frequency f)
+// Word f / 32 of a frequency bitmap for a lane-dependent f.  The bitmaps are kernel arguments: indexed per lane they
+// would be fetched from the argument segment with a vector load, one more memory round trip between a wave's
+// positions and its table loads.  The words are pinned in scalar registers instead and picked with selects.
+template <int D>
+__device__ __forceinline__ uint32_t bitmap_word(const uint32_t (&bitmap)[4], int f) {
+    uint32_t w0 = bitmap[0], w1 = bitmap[1], w2 = bitmap[2], w3 = bitmap[3];
+    if constexpr (D / 2 <= 32) {
+        asm("" : "+s"(w0));
+        return w0;
+    } else if constexpr (D / 2 <= 64) {
+        asm("" : "+s"(w0), "+s"(w1));
+        return f < 32 ? w0 : w1;
+    } else {
+        asm("" : "+s"(w0), "+s"(w1), "+s"(w2), "+s"(w3));
+        return f < 64 ? (f < 32 ? w0 : w1) : (f < 96 ? w2 : w3);
+    }
+}
 template <int D, bool NEOX>
 __device__ __forceinline__ uint32_t trig_bits(const uint32_t (&bitmap)[4], int sub) {
     if constexpr (NEOX) {
         const int f = 8 * sub;
-        return (bitmap[f >> 5] >> (f & 31)) & 0xffu;
+        return (bitmap_word<D>(bitmap, f) >> (f & 31)) & 0xffu;
     } else {
         const int f0 = 4 * sub, f1 = D / 4 + 4 * sub;
-        return ((bitmap[f0 >> 5] >> (f0 & 31)) & 0xfu) | (((bitmap[f1 >> 5] >> (f1 & 31)) & 0xfu) << 4);
+        return ((bitmap_word<D>(bitmap, f0) >> (f0 & 31)) & 0xfu) | (((bitmap_word<D>(bitmap, f1) >> (f1 & 31)) & 0xfu) << 4);
     }
 }
 
@@ -206,6 +223,14 @@ struct RopeUnit {
     static __device__ __forceinline__ void issue_loads(const RopeArgs &a, uint32_t unit, int lane, UnitState &st) {
         st.live = unit < a.total_units;  // wave-uniform
         if (!st.live) return;
+        // With three position axes both weight pointers are pinned in scalar registers, here, ahead of every other
+        // load: the select between the two kernel arguments is otherwise turned into a per-lane load of the pointer
+        // from the argument segment in those instantiations, and the weights wait for that round trip (30.0 -> 27.0
+        // us at 8192 tokens of 28+4 heads, together with the bitmap words of trig_bits).  The one-axis instantiations
+        // keep the pointers in scalar registers by themselves and lose 2-7 % to the pin.  (Not volatile: a volatile
+        // statement ahead of them turns the position loads into vector loads.)
+        const void *qw = a.qw, *kw = a.kw;
+        if constexpr (AXES == 3) asm("" : "+s"(qw), "+s"(kw));
         st.t = a.upt_magic ? __umulhi(unit, a.upt_magic) : unit;
         st.u = unit - st.t * a.units_per_token;
         const int sub = lane % LPH, hl = lane / LPH;
@@ -236,7 +261,7 @@ struct RopeUnit {
                 st.vchunk = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(st.token_in + (int64_t)heads_qk * D + 8 * v_first));
         }
 
-        const uint16_t *wsrc = static_cast<const uint16_t *>(st.is_q ? a.qw : a.kw);
+        const uint16_t *wsrc = static_cast<const uint16_t *>(st.is_q ? qw : kw);
         st.wa = *reinterpret_cast<const u32x4 *>(wsrc + c0(sub));
         st.wb = *reinterpret_cast<const u32x4 *>(wsrc + c1(sub));
 
@@ -1132,16 +1157,15 @@ int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allo
 //                      chip's 1024 SIMDs, so its run time moves in steps of ceil(waves / 1024) waves per SIMD (one
 //                      token per wave, 40 heads: 9.2 us at 1024 tokens, 12.1 at 2048, 15.4 at 3072, 19.0 at 4096,
 //                      and 14.5-14.8 anywhere from 2400 to 2800) while the other kernel's grows with the tokens.
-//                      Against the other kernel with streaming stores it is ahead where its last step is full and
-//                      three or four waves sit on every SIMD, and then only (a) with three position axes, where a
-//                      token's merged table row is fetched once instead of three rows per group of heads (28+4
-//                      heads: 16.3 against 17.5 us at 4096 tokens, 21.5 against 24.1 at 6144, 28.0 against 30.2 at
-//                      8192, 52.1 against 54.8 at 16384; 3-4 % with an fp8 cache), and (b) with one axis, a 16-bit
-//                      cache and one token per wave (40 heads of 128: 18.45 against 18.9 us at 4096 tokens, 14.9
-//                      against 15.1 at 3072).  Elsewhere the other kernel is level or ahead: 33.9 against 35.1 us at
-//                      8192 x 40 heads, 65.1 against 68.6 at 16384, 28.0 against 31.5 at 4096 x 72 heads with an fp8
-//                      cache, 65.6 against 70.7 at 8192 x 40 heads of 256, and by 10 % where the walking grid's last
-//                      step is thin (19.2 against 22.8 us at 4100 tokens);
+//                      Against the other kernel with streaming stores it is ahead only with one position axis, a
+//                      16-bit cache, head size 128 and one token per wave on a grid whose last step is full with three
+//                      or four waves on every SIMD (40 heads: 18.45 against 18.9 us at 4096 tokens, 14.9 against 15.1
+//                      at 3072; in place 15.9 against 16.6).  Elsewhere the other kernel is level or ahead: 33.6
+//                      against 35.8 us at 8192 x 40 heads, 64.8 against 69.0 at 16384, 28.0 against 31.5 at 4096 x 72
+//                      heads with an fp8 cache, 65.6 against 70.7 at 8192 x 40 heads of 256, with three position axes
+//                      27.0 against 27.7 at 8192 x 32 heads and 50.7 against 51.9 at 16384 (16.5 both at 4096 with
+//                      an fp8 cache), and by 10-20 % where the walking grid's last step is thin (19.1 against 22.9 us
+//                      at 4100 tokens);
 //   one wave per unit: everything else.
 // (Cutting a token's units into runs shared by neighbouring waves, to fill the slots at any T, was measured too: it
 // narrows the walking kernel's dips -- 22.1 us at 4608 -- but never beats the better of the two kernels.)
@@ -1163,7 +1187,7 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
     const uint32_t simds = 4 * kComputeUnits;
     const uint32_t waves_per_simd = (walk_waves + simds - 1) / simds;  // of the fullest SIMD
     const bool last_step_full = waves_per_simd >= 3 && 100 * (uint64_t)walk_waves >= 95 * (uint64_t)waves_per_simd * simds;
-    const bool slots_filled = last_step_full && (AXES == 3 || (!KVFP8 && D == 128 && tokens_per_wave == 1));
+    const bool slots_filled = last_step_full && AXES == 1 && !KVFP8 && D == 128 && tokens_per_wave == 1;
     const bool walk = v_fits && strides_fit &&
                       (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits && slots_filled));
     RopeArgs b = a;

@@ -259,10 +259,9 @@ def test_token_walking_kernel(device, case, waves, stream):
 
 
 def test_kernel_choice_by_batch_size(device):
-    """The built-in rule: the walking kernel where three or four of its waves sit on nearly every SIMD (2920-3072 and
-    3892-4096 tokens with one token per wave; the same bands of tokens / tokens per wave above), and then only with
-    three position axes or, with one axis, a 16-bit cache and one token per wave; the one-wave-per-unit kernel
-    elsewhere, with its q_out / K rows streamed past the L2 from 8 MB per call on.  All of them meet the oracle (sizes
+    """The built-in rule: the walking kernel where three or four of its waves sit on nearly every SIMD with one token
+    each (2920-3072 and 3892-4096 tokens), and then only with one position axis, a 16-bit cache and head size 128; the
+    one-wave-per-unit kernel elsewhere, with its q_out / K rows streamed past the L2 from 8 MB per call on.  All of them meet the oracle (sizes
     on both sides of each switch; mRoPE and plain RoPE; an fp8 cache; too many V heads for the walking kernel)."""
     cases = ((2900, (32, 8, 8), False, False), (3000, (32, 8, 8), False, False), (4100, (32, 8, 8), False, False),
              (6100, (12, 4, 4), False, True), (5800, (12, 4, 4), False, True), (4000, (12, 4, 4), True, False),
