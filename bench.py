@@ -337,13 +337,22 @@ def main():
             avg, med, mn = per_launch_ms(call, 100)
             return nbytes, avg, med, mn, burst
 
+        def rope_kernel_label(r):
+            # what the launcher picks for this batch, asked of the library
+            walking, groups, lanes, streamed = capi.rope_rms_launch_shape(
+                r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
+                3 if r.mrope_section is not None else 1, torch.bfloat16, True, r.kv_dtype == torch.float8_e4m3fn)
+            form = ("rope_rms_walk_kernel (one wave per token or run of tokens)" if walking
+                    else "rope_rms_kernel (one wave per group of heads)")
+            return f"{form}, {groups} workgroups x {lanes} lanes, rows stored {'past the L2' if streamed else 'through the L2'}"
+
         for name, r in (("rope_kv_qwen3_T4096", workloads.config3()), ("mrope_kv_qwen2vl_T8192", workloads.config4())):
             nbytes, avg, med, mn, burst = rope_case(r, 4)
             extras[name] = {"us_per_call": round(burst * 1e3, 2), "avg_launch_us": round(avg * 1e3, 2),
                             "GBps": round(nbytes / (burst * 1e-3) / 1e9, 1),
                             "frac_of_8TBps": round(nbytes / (burst * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                             "algorithmic_bytes": nbytes, "copy_same_bytes_us": copy_same_bytes_us(nbytes),
-                            "kernel": "rope_rms_walk_kernel (token-walking, one dispatch round of up to 4096 waves)"}
+                            "kernel": rope_kernel_label(r)}
         del src, dst
 
         # the two-stream op at the reference script's shape (test/test_fused_rope_rms_2way.py:223-246), and the no-KV

@@ -15,7 +15,8 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "lib
 
 EXPORTS = ("gpuk_status_string", "gpuk_abi_version", "gpuk_add_rmsnorm_quant", "gpuk_rope_rms",
            "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_increment_floats", "gpuk_set_tuning",
-           "gpuk_add_rmsnorm_quant_traffic_only", "gpuk_add_rmsnorm_quant_launch_shape")
+           "gpuk_add_rmsnorm_quant_traffic_only", "gpuk_add_rmsnorm_quant_launch_shape",
+           "gpuk_rope_rms_launch_shape")
 
 DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2, torch.float64: 3}
 QUANT_NONE, QUANT_FP8_DYNAMIC, QUANT_FP8_E4M3FNUZ, QUANT_FP8_STATIC = 0, 1, 2, 3
@@ -60,6 +61,8 @@ def lib():
         L.gpuk_add_rmsnorm_quant_traffic_only.argtypes = [C.c_void_p] * 5 + [C.c_int64, C.c_int64, C.c_void_p]
         L.gpuk_add_rmsnorm_quant_launch_shape.restype = C.c_int
         L.gpuk_add_rmsnorm_quant_launch_shape.argtypes = [C.c_int64, C.c_int64, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        L.gpuk_rope_rms_launch_shape.restype = C.c_int
+        L.gpuk_rope_rms_launch_shape.argtypes = [C.c_int64] * 5 + [C.c_int] * 4 + [C.POINTER(C.c_int)] * 4
         L.gpuk_copy_bytes.restype = C.c_int
         L.gpuk_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
         _lib = L
@@ -107,6 +110,17 @@ def add_rmsnorm_quant_launch_shape(tokens: int, hidden: int, dtype=torch.bfloat1
     if rc:
         raise GpukError(rc, "gpuk_add_rmsnorm_quant_launch_shape")
     return lanes.value, chunks.value
+
+
+def rope_rms_launch_shape(num_tokens: int, num_heads_q: int, num_heads_k: int, num_heads_v: int, head_size: int,
+                          n_axes: int = 1, dtype=torch.bfloat16, set_kv: bool = True, kv_fp8: bool = False):
+    """(walking, workgroups, lanes per workgroup, streamed) of the launch the rope entry points make for this batch."""
+    out = [C.c_int(0) for _ in range(4)]
+    rc = lib().gpuk_rope_rms_launch_shape(num_tokens, num_heads_q, num_heads_k, num_heads_v, head_size, n_axes,
+                                          DTYPE[dtype], int(set_kv), 1 if kv_fp8 else 0, *(C.byref(o) for o in out))
+    if rc:
+        raise GpukError(rc, "gpuk_rope_rms_launch_shape")
+    return bool(out[0].value), out[1].value, out[2].value, bool(out[3].value)
 
 
 def _pos_args(positions):

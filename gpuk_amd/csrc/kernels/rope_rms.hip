@@ -1175,45 +1175,65 @@ constexpr int64_t kUnitStreamBytes = 8'000'000;
 constexpr uint32_t kWalkCapacity = 4096;  // waves the chip holds at once at 4 per SIMD: one dispatch round
 constexpr uint32_t kComputeUnits = 256;   // MI355X
 
-template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
-int launch_one(const RopeArgs &a, hipStream_t stream) {
+// What a call of the 16-bit rope kernels launches: which kernel, its grid, whether the output rows go past the L2.
+struct RopePlan {
+    bool walk;                  // token-walking kernel (else one wave per unit)
+    uint32_t walk_waves;        // its grid, in waves
+    uint32_t threads, blocks;   // workgroup size and count of the launch
+    bool stream;                // q_out / K rows / in-place rows stored past the L2
+};
+
+RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8) {
+    RopePlan p{};
     // the walking kernel shares a token's V row out over the token's units, one 16-byte chunk per lane and unit
-    const bool v_fits = !SETKV || (int64_t)a.units_per_token * 64 >= (int64_t)a.hv * (D / 8);
+    const bool v_fits = !set_kv || (int64_t)a.units_per_token * 64 >= (int64_t)a.hv * (D / 8);
     const bool strides_fit = a.ps_token == (int)a.ps_token && a.ps_axis == (int)a.ps_axis;  // passed as 32-bit
     // every wave the same number of tokens (the last ones one fewer)
     const uint32_t capacity = g_walk_waves ? (uint32_t)g_walk_waves : kWalkCapacity;
     const uint32_t tokens_per_wave = (a.num_tokens + capacity - 1) / capacity;
-    const uint32_t walk_waves = (a.num_tokens + tokens_per_wave - 1) / tokens_per_wave;
+    p.walk_waves = (a.num_tokens + tokens_per_wave - 1) / tokens_per_wave;
     const uint32_t simds = 4 * kComputeUnits;
-    const uint32_t waves_per_simd = (walk_waves + simds - 1) / simds;  // of the fullest SIMD
-    const bool last_step_full = waves_per_simd >= 3 && 100 * (uint64_t)walk_waves >= 95 * (uint64_t)waves_per_simd * simds;
-    const bool slots_filled = last_step_full && AXES == 1 && !KVFP8 && D == 128 && tokens_per_wave == 1;
-    const bool walk = v_fits && strides_fit &&
-                      (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits && slots_filled));
-    RopeArgs b = a;
+    const uint32_t waves_per_simd = (p.walk_waves + simds - 1) / simds;  // of the fullest SIMD
+    const bool last_step_full = waves_per_simd >= 3 && 100 * (uint64_t)p.walk_waves >= 95 * (uint64_t)waves_per_simd * simds;
+    const bool slots_filled = last_step_full && axes == 1 && !kv_fp8 && D == 128 && tokens_per_wave == 1;
+    p.walk = v_fits && strides_fit &&
+             (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits && slots_filled));
     // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
     const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
-    const int64_t call_bytes = SETKV ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
-                                           (KVFP8 ? 1 : 2) * ((int64_t)a.num_tokens * a.hk * D + elems_v)
-                                     : 4 * elems_qk;
-    const int64_t stream_from = walk ? kWalkStreamBytes : kUnitStreamBytes;
-    b.walk_stream = g_walk_stream == 2 || (g_walk_stream == 0 && call_bytes >= stream_from) ? 1u : 0u;
-    if (walk) {
-        b.walk_waves = walk_waves;
-        rope_rms_walk_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<(b.walk_waves + kWalkWaves - 1) / kWalkWaves, kWalkWaves * 64, 0, stream>>>(
+    const int64_t call_bytes = set_kv ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
+                                            (kv_fp8 ? 1 : 2) * ((int64_t)a.num_tokens * a.hk * D + elems_v)
+                                      : 4 * elems_qk;
+    const int64_t stream_from = p.walk ? kWalkStreamBytes : kUnitStreamBytes;
+    p.stream = g_walk_stream == 2 || (g_walk_stream == 0 && call_bytes >= stream_from);
+    if (p.walk) {
+        p.threads = kWalkWaves * 64;
+        p.blocks = (p.walk_waves + kWalkWaves - 1) / kWalkWaves;
+    } else {
+        // Workgroup size, swept over 64/128/256/512 lanes and one workgroup per token for 2-9 units per token: four
+        // waves where a workgroup then holds whole tokens (its waves share the token's position and table row in the
+        // CU's caches: 3-15 % ahead at 28+4 heads) and for large batches (1-3 % ahead from 4096 tokens on), single
+        // waves for small batches of other head counts (2-6 % ahead at 64+8 heads with an fp8 cache up to 512 tokens,
+        // within 1-3 % either way for 3, 5 and 6 units per token); 128 lanes is the slowest in most cases.
+        p.threads = g_block_threads ? (uint32_t)g_block_threads : (a.units_per_token % 4 == 0 || a.total_units > 8192 ? 256u : 64u);
+        const uint32_t units_per_block = p.threads / 64;
+        p.blocks = (a.total_units + units_per_block - 1) / units_per_block;
+    }
+    return p;
+}
+
+template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
+int launch_one(const RopeArgs &a, hipStream_t stream) {
+    const RopePlan p = plan_rope(a, D, AXES, SETKV, KVFP8);
+    RopeArgs b = a;
+    b.walk_stream = p.stream ? 1u : 0u;
+    if (p.walk) {
+        b.walk_waves = p.walk_waves;
+        rope_rms_walk_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<p.blocks, p.threads, 0, stream>>>(
             a.positions, a.kv_loc, a.qkv_in, a.cos_sin, b.walk_waves, a.num_tokens, a.units_per_token, a.hq + a.hk,
             a.hq + a.hk + a.hv, (int)a.ps_token, (int)a.ps_axis, a.hv, b);
         return hip_status(hipGetLastError());
     }
-    // Workgroup size, swept over 64/128/256/512 lanes and one workgroup per token for 2-9 units per token: four waves
-    // where a workgroup then holds whole tokens (its waves share the token's position and table row in the CU's
-    // caches: 3-15 % ahead at 28+4 heads) and for large batches (1-3 % ahead from 4096 tokens on), single waves for
-    // small batches of other head counts (2-6 % ahead at 64+8 heads with an fp8 cache up to 512 tokens, within 1-3 %
-    // either way for 3, 5 and 6 units per token); 128 lanes is the slowest in most cases.
-    const int threads = g_block_threads ? g_block_threads : (a.units_per_token % 4 == 0 || a.total_units > 8192 ? 256 : 64);
-    const uint32_t units_per_block = threads / 64;
-    const uint32_t blocks = (a.total_units + units_per_block - 1) / units_per_block;
-    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<blocks, threads, 0, stream>>>(b);
+    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<p.blocks, p.threads, 0, stream>>>(b);
     return hip_status(hipGetLastError());
 }
 
@@ -1363,6 +1383,38 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     return launch_head_size<FP16>(a, D, neox != 0, n_axes, set_kv, kv_fp8, s);
 }
 
+int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, int n_axes, int dtype, bool set_kv,
+                      int kv_dtype, int *walking, int *workgroups, int *lanes, int *streamed) {
+    if (T <= 0 || hq < 0 || hk < 0 || hv < 0 || hq + hk == 0 || (n_axes != 1 && n_axes != 3)) return GPUK_ERR_INVALID_ARG;
+    if (D != 64 && D != 128 && D != 256) return GPUK_ERR_UNSUPPORTED;
+    if (!walking || !workgroups || !lanes || !streamed) return GPUK_ERR_INVALID_ARG;
+    const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
+    const int64_t hpw = 64 / (D / 16);
+    const int64_t upt = wide ? hq + hk + (set_kv ? hv : 0) : (hq + hk + hpw - 1) / hpw;
+    if (upt * T >= 0x7fffffffLL || upt * T * upt >= (1LL << 32)) return GPUK_ERR_UNSUPPORTED;
+    RopeArgs a{};
+    a.total_units = (uint32_t)(upt * T);
+    a.num_tokens = (uint32_t)T;
+    a.units_per_token = (uint32_t)upt;
+    a.hq = (int)hq;
+    a.hk = (int)hk;
+    a.hv = (int)hv;
+    a.ps_token = 1;  // positions as the wrappers pass them: strides that fit 32 bits
+    if (wide) {
+        *walking = 0;
+        *workgroups = (int)((a.total_units + 3) / 4);
+        *lanes = 256;
+        *streamed = 0;
+        return GPUK_OK;
+    }
+    const RopePlan p = plan_rope(a, (int)D, n_axes, set_kv, set_kv && kv_dtype == GPUK_KV_E4M3FN);
+    *walking = p.walk ? 1 : 0;
+    *workgroups = (int)p.blocks;
+    *lanes = (int)p.threads;
+    *streamed = p.stream ? 1 : 0;
+    return GPUK_OK;
+}
+
 }  // namespace
 
 void set_rope_tuning(int key, int value) {
@@ -1374,6 +1426,14 @@ void set_rope_tuning(int key, int value) {
 }
 
 }  // namespace gpuk
+
+extern "C" int gpuk_rope_rms_launch_shape(int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k,
+                                          int64_t num_heads_v, int64_t head_size, int n_axes, int dtype, int set_kv,
+                                          int kv_dtype, int *walking, int *workgroups, int *lanes_per_workgroup,
+                                          int *streamed) {
+    return gpuk::rope_launch_shape(num_tokens, num_heads_q, num_heads_k, num_heads_v, head_size, n_axes, dtype,
+                                   set_kv != 0, kv_dtype, walking, workgroups, lanes_per_workgroup, streamed);
+}
 
 extern "C" int gpuk_rope_rms(void *qkv, const void *qw, const void *kw, const void *cos_sin, const int64_t *positions,
                              int64_t pos_stride_axis, int64_t pos_stride_token, int n_axes, int64_t num_tokens,

@@ -178,6 +178,17 @@ int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidden, int dtyp
                                         int *chunks_per_lane);
 
 /*
+ * The launch gpuk_rope_rms_set_kv (set_kv != 0) or gpuk_rope_rms (set_kv == 0) makes for a batch with contiguous
+ * positions: *walking = 1 for the token-walking kernel (one wave per token or run of tokens), 0 for the kernel with
+ * one wave per group of heads; the grid as workgroups x lanes per workgroup; *streamed = 1 when the rotated rows are
+ * stored past the L2.  Computed on the host from the sizes and the tuning keys; the four outputs are host pointers.
+ * For reports.  Not part of the reference.
+ */
+int gpuk_rope_rms_launch_shape(int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                               int64_t head_size, int n_axes, int dtype, int set_kv, int kv_dtype, int *walking,
+                               int *workgroups, int *lanes_per_workgroup, int *streamed);
+
+/*
  * Launch-cost calibration: data[i] += 1 for i in [0, n) (data 16-byte aligned).  With a small n the call costs
  * what launching and draining any kernel costs, the floor under decode-sized calls.
  * Counterpart of the reference's micro-benchmark test/cpp/test_small_kernel.cpp:85-126.

@@ -266,3 +266,28 @@ def test_launch_shape_report():
     assert L.gpuk_add_rmsnorm_quant_launch_shape(0, 1024, 0, C.byref(a), C.byref(b)) == 1
     assert L.gpuk_add_rmsnorm_quant_launch_shape(4, 1027, 0, C.byref(a), C.byref(b)) == 2
     assert L.gpuk_add_rmsnorm_quant_launch_shape(4, 1024, 0, None, C.byref(b)) == 1
+
+
+def test_rope_launch_shape_report():
+    """gpuk_rope_rms_launch_shape computes on the host which rope kernel a batch gets, its grid and whether the rotated
+    rows are stored past the L2; no GPU is needed."""
+    from gpuk_amd import capi
+    # 4096 tokens x (32, 8, 8) heads of 128: one wave per token fills every SIMD four times -> the walking kernel
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128) == (True, 1024, 256, False)
+    # three position axes, or an fp8 cache: one wave per group of 8 heads, four waves a workgroup, streamed stores
+    assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3) == (False, 8192, 256, True)
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (False, 5120, 256, True)
+    # a decode batch: single waves, through the L2
+    assert capi.rope_rms_launch_shape(16, 28, 4, 4, 128) == (False, 16, 256, False)
+    assert capi.rope_rms_launch_shape(16, 40, 8, 8, 128, kv_fp8=True) == (False, 96, 64, False)
+    # fp32 activations: one wave per head, V heads included when a cache is written
+    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32) == (False, 20, 256, False)
+    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32, set_kv=False) == (False, 15, 256, False)
+    import ctypes as C
+    L = capi.lib()
+    o = [C.c_int(0) for _ in range(4)]
+    refs = [C.byref(x) for x in o]
+    assert L.gpuk_rope_rms_launch_shape(0, 32, 8, 8, 128, 1, 0, 1, 0, *refs) == 1
+    assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 96, 1, 0, 1, 0, *refs) == 2
+    assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 128, 2, 0, 1, 0, *refs) == 1
+    assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 128, 1, 0, 1, 0, None, *refs[1:]) == 1
