@@ -323,16 +323,17 @@ add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict
 }
 
 // fp32 and fp64 activations: the reference dispatches them through the same template
-// (AT_DISPATCH_FLOATING_TYPES_AND2, src/ops/all_reduce_fusion.cpp:375-378).  A compatibility path, not a tuned one:
-// three sweeps over the row like the long-row kernel, 4 elements per chunk.  Rounding to the activation type is the
-// identity here, so the oracle's sequence is plain arithmetic in that type around an fp32 variance:
+// (AT_DISPATCH_FLOATING_TYPES_AND2, src/ops/all_reduce_fusion.cpp:375-378).  4 elements per chunk; a lane keeps its
+// CPL chunks of the summed row in registers (rows of up to 4 x 1024 chunks), or, with CPL = 0, sweeps a longer row
+// three times, reading back what it stored to residual_out.  Rounding to the activation type is the identity here, so
+// the oracle's sequence is plain arithmetic in that type around an fp32 variance:
 //   res = x + r;  rstd = 1/sqrt(mean(float(res)^2) + eps) in fp32;  n = gamma * (res * F(rstd));
 //   scale = max|float(n)| / fp8_max in fp32;  code = e4m3fn(float(clamp(n / F(scale))))
 // (for F = double torch promotes tensor * fp32-tensor products to double and casts double -> float -> fp8).
 template <typename F>
 using wide4 = F __attribute__((ext_vector_type(4)));
 
-template <typename F, int QUANT>
+template <typename F, int QUANT, int CPL>
 __global__ void __launch_bounds__(kMaxThreads)
 add_rmsnorm_quant_wide_rows(const wide4<F> *__restrict__ x, const wide4<F> *__restrict__ residual_in,
                             const wide4<F> *__restrict__ gamma, wide4<F> *residual_out, void *__restrict__ norm_out,
@@ -342,38 +343,67 @@ add_rmsnorm_quant_wide_rows(const wide4<F> *__restrict__ x, const wide4<F> *__re
     const int tid = threadIdx.x;
     const int num_waves = blockDim.x >> 6;
     const int64_t row_base = (int64_t)blockIdx.x * chunks_per_row;
+    constexpr int KEPT = CPL ? CPL : 1;
+    // streaming accesses where the row stays in registers: measured 6-12 % faster for fp32 and 12 % slower for fp64
+    constexpr bool STREAM = CPL > 0 && sizeof(F) == 4;
+    wide4<F> kept[KEPT];  // CPL > 0: chunk tid + i * blockDim.x of the summed row (and later of the normed row)
+
+    // f(i, c) for every chunk c of the row this lane owns; i is its place in kept[]
+    auto for_chunks = [&](auto f) {
+        if constexpr (CPL > 0) {
+#pragma unroll
+            for (int i = 0; i < CPL; ++i) {
+                const int c = tid + i * (int)blockDim.x;
+                if (c < chunks_per_row) f(i, c);
+            }
+        } else {
+            for (int c = tid; c < chunks_per_row; c += blockDim.x) f(0, c);
+        }
+    };
 
     float ss = 0.f;
-    for (int c = tid; c < chunks_per_row; c += blockDim.x) {
-        const wide4<F> res = x[row_base + c] + residual_in[row_base + c];
-        residual_out[row_base + c] = res;
+    for_chunks([&](int i, int c) {
+        wide4<F> res;
+        if constexpr (STREAM) {
+            res = __builtin_nontemporal_load(x + row_base + c) + __builtin_nontemporal_load(residual_in + row_base + c);
+            __builtin_nontemporal_store(res, residual_out + row_base + c);
+        } else {
+            res = x[row_base + c] + residual_in[row_base + c];
+            residual_out[row_base + c] = res;  // CPL = 0: read back below
+        }
+        kept[i] = res;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const float r = (float)res[j];
             ss = __builtin_fmaf(r, r, ss);
         }
-    }
+    });
     float sumsq[1] = {ss};
     block_allreduce<SumOp, 1>(sumsq, s_sum, num_waves);
     const F rstd = (F)(1.0f / sqrtf(sumsq[0] / hidden_f + eps));
 
-    auto normed = [&](int c) {
-        const wide4<F> v = residual_out[row_base + c];  // written by this lane above
+    // the normed chunk; with CPL = 0 the summed chunk is read back (this lane wrote it above)
+    auto normed = [&](int i, int c) {
+        const wide4<F> v = CPL > 0 ? kept[i] : residual_out[row_base + c];
         return gamma[c] * (v * rstd);
     };
 
     if constexpr (QUANT == GPUK_QUANT_NONE) {
         wide4<F> *out = reinterpret_cast<wide4<F> *>(norm_out) + row_base;
-        for (int c = tid; c < chunks_per_row; c += blockDim.x) out[c] = normed(c);
+        for_chunks([&](int i, int c) {
+            if constexpr (STREAM) __builtin_nontemporal_store(normed(i, c), out + c);
+            else out[c] = normed(i, c);
+        });
     } else {
         float scale;
         if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
             float amax = 0.f;
-            for (int c = tid; c < chunks_per_row; c += blockDim.x) {
-                const wide4<F> v = normed(c);
+            for_chunks([&](int i, int c) {
+                const wide4<F> v = normed(i, c);
+                if constexpr (CPL > 0) kept[i] = v;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) amax = MaxOp::apply(amax, __builtin_fabsf((float)v[j]));
-            }
+            });
             float am[1] = {amax};
             block_allreduce<MaxOp, 1>(am, s_max, num_waves);
             scale = am[0] == 0.f ? 1.f : am[0] / fp8_max;
@@ -383,12 +413,17 @@ add_rmsnorm_quant_wide_rows(const wide4<F> *__restrict__ x, const wide4<F> *__re
         }
         const F wide_scale = (F)scale;
         uint32_t *out = reinterpret_cast<uint32_t *>(norm_out) + row_base;
-        for (int c = tid; c < chunks_per_row; c += blockDim.x) {
-            const wide4<F> q = normed(c) / wide_scale;
+        for_chunks([&](int i, int c) {
+            wide4<F> n;
+            if constexpr (CPL > 0 && QUANT == GPUK_QUANT_FP8_DYNAMIC) n = kept[i];
+            else n = normed(i, c);
+            const wide4<F> q = n / wide_scale;
             // clamping after the cast to fp32 equals the oracle's clamp before it: the bounds are fp32 numbers
-            out[c] = cvt4_e4m3fn(clamp_sym((float)q[0], fp8_max), clamp_sym((float)q[1], fp8_max),
-                                 clamp_sym((float)q[2], fp8_max), clamp_sym((float)q[3], fp8_max));
-        }
+            const uint32_t codes = cvt4_e4m3fn(clamp_sym((float)q[0], fp8_max), clamp_sym((float)q[1], fp8_max),
+                                               clamp_sym((float)q[2], fp8_max), clamp_sym((float)q[3], fp8_max));
+            if constexpr (STREAM) __builtin_nontemporal_store(codes, out + c);
+            else out[c] = codes;
+        });
     }
 }
 
@@ -464,15 +499,40 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
     return hip_status(hipGetLastError());
 }
 
+// Lanes and kept chunks per lane of the fp32 / fp64 kernel; 0 chunks kept = rows beyond 4096 chunks, swept.  fp32, as
+// for the 16-bit kernel: two chunks per lane unless that leaves more lanes idle in the last wave (12 % ahead of one
+// chunk at 32768 x 4096); fp64: one chunk (32 bytes) per lane up to 1024 lanes (6 % ahead of two).
+void pick_wide_shape(int chunks, bool fp64, int *threads, int *cpl) {
+    const int lanes1 = round_up(chunks, 64), lanes2 = round_up((chunks + 1) / 2, 64);
+    int n = (fp64 || 2 * lanes2 > lanes1) && lanes1 <= kMaxThreads ? 1 : 2;
+    while (n < 4 && chunks > n * kMaxThreads) n *= 2;
+    if (chunks > n * kMaxThreads) {
+        *cpl = 0;
+        *threads = kMaxThreads;
+        return;
+    }
+    *cpl = n;
+    *threads = round_up((chunks + n - 1) / n, 64);
+}
+
 template <typename F, int QUANT>
 int launch_wide(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
                 float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream) {
     const int chunks = (int)(hidden / 4);
-    const int want = (chunks + 63) / 64 * 64;
-    const int threads = want < kMaxThreads ? want : kMaxThreads;
-    add_rmsnorm_quant_wide_rows<F, QUANT><<<dim3((unsigned)tokens), threads, 0, stream>>>(
-        static_cast<const wide4<F> *>(x), static_cast<const wide4<F> *>(residual_in), static_cast<const wide4<F> *>(gamma),
-        static_cast<wide4<F> *>(residual_out), norm_out, scale, chunks, (float)hidden, eps, fp8_max);
+    int threads, cpl;
+    pick_wide_shape(chunks, sizeof(F) == 8, &threads, &cpl);
+#define GPUK_LAUNCH_WIDE(CPL)                                                                                          \
+    add_rmsnorm_quant_wide_rows<F, QUANT, CPL><<<dim3((unsigned)tokens), threads, 0, stream>>>(                        \
+        static_cast<const wide4<F> *>(x), static_cast<const wide4<F> *>(residual_in),                                  \
+        static_cast<const wide4<F> *>(gamma), static_cast<wide4<F> *>(residual_out), norm_out, scale, chunks,          \
+        (float)hidden, eps, fp8_max)
+    switch (cpl) {
+        case 1: GPUK_LAUNCH_WIDE(1); break;
+        case 2: GPUK_LAUNCH_WIDE(2); break;
+        case 4: GPUK_LAUNCH_WIDE(4); break;
+        default: GPUK_LAUNCH_WIDE(0); break;
+    }
+#undef GPUK_LAUNCH_WIDE
     return hip_status(hipGetLastError());
 }
 
@@ -553,10 +613,8 @@ extern "C" int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidde
     const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
     const int elems = wide ? 4 : 8;
     if (hidden % elems != 0) return GPUK_ERR_UNSUPPORTED;
-    if (wide) {  // the fp32 / fp64 path sweeps the row: lanes only
-        const int want = ((int)(hidden / 4) + 63) / 64 * 64;
-        *lanes_per_row = want < kMaxThreads ? want : kMaxThreads;
-        *chunks_per_lane = 0;
+    if (wide) {  // the fp32 / fp64 kernel: 4-element chunks, 0 = rows swept three times
+        pick_wide_shape((int)(hidden / 4), dtype == GPUK_DTYPE_F64, lanes_per_row, chunks_per_lane);
         return GPUK_OK;
     }
     pick_shape(tokens, (int)(hidden / 8), lanes_per_row, chunks_per_lane);

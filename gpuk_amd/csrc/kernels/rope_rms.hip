@@ -924,26 +924,8 @@ __global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
 
     const bool is_q = h < a.hq;
     const F *w = static_cast<const F *>(is_q ? a.qw : a.kw);
-    F x1[PPL], x2[PPL];
-    int i1[PPL], i2[PPL];
-    bool live[PPL];
-    float ss = 0.f;
-#pragma unroll
-    for (int k = 0; k < PPL; ++k) {
-        const int p = lane + 64 * k;
-        live[k] = p < HALF;
-        const int pc = live[k] ? p : 0;
-        i1[k] = NEOX ? pc : 2 * pc;
-        i2[k] = NEOX ? pc + HALF : 2 * pc + 1;
-        x1[k] = live[k] ? src[i1[k]] : (F)0;
-        x2[k] = live[k] ? src[i2[k]] : (F)0;
-        const float f1 = (float)x1[k], f2 = (float)x2[k];
-        ss = __builtin_fmaf(f1, f1, ss);
-        ss = __builtin_fmaf(f2, f2, ss);
-    }
-    ss = wave_allreduce<SumOp>(ss);
-    const F rstd = (F)(1.0f / sqrtf(ss * (1.0f / D) + a.eps));
-
+    // every load of the wave is issued before the first use: positions and slot (wave-uniform), then x, weights and
+    // the cos/sin values, whose rows depend on the positions
     const F *table = static_cast<const F *>(a.cos_sin);
     const int64_t p0 = a.positions[(int64_t)t * a.ps_token];
     int64_t p1 = p0, p2 = p0;
@@ -951,6 +933,40 @@ __global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
         p1 = a.positions[a.ps_axis + (int64_t)t * a.ps_token];
         p2 = a.positions[2 * a.ps_axis + (int64_t)t * a.ps_token];
     }
+    int64_t slot = 0;
+    if constexpr (SETKV) slot = a.kv_loc[t];
+    F x1[PPL], x2[PPL], w1[PPL], w2[PPL], c[PPL], s[PPL];
+    int i1[PPL], i2[PPL];
+    bool live[PPL];
+#pragma unroll
+    for (int k = 0; k < PPL; ++k) {
+        const int f = lane + 64 * k;  // rotary frequency of this pair
+        live[k] = f < HALF;
+        const int fc = live[k] ? f : 0;
+        i1[k] = NEOX ? fc : 2 * fc;
+        i2[k] = NEOX ? fc + HALF : 2 * fc + 1;
+        x1[k] = live[k] ? src[i1[k]] : (F)0;
+        x2[k] = live[k] ? src[i2[k]] : (F)0;
+        w1[k] = w[i1[k]];
+        w2[k] = w[i2[k]];
+        int64_t pos = p0;
+        if constexpr (AXES == 3) {
+            const bool on1 = (a.axis1[fc >> 5] >> (fc & 31)) & 1u, on2 = (a.axis2[fc >> 5] >> (fc & 31)) & 1u;
+            pos = on2 ? p2 : (on1 ? p1 : p0);
+        }
+        c[k] = table[pos * D + fc];
+        s[k] = table[pos * D + HALF + fc];
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < PPL; ++k) {
+        const float f1 = (float)x1[k], f2 = (float)x2[k];
+        ss = __builtin_fmaf(f1, f1, ss);
+        ss = __builtin_fmaf(f2, f2, ss);
+    }
+    ss = wave_allreduce<SumOp>(ss);
+    const F rstd = (F)(1.0f / sqrtf(ss * (1.0f / D) + a.eps));
+
     F *dst;
     uint8_t *dst8 = nullptr;
     if constexpr (!SETKV) {
@@ -958,7 +974,6 @@ __global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
     } else if (is_q) {
         dst = static_cast<F *>(a.q_out) + ((int64_t)t * a.hq + h) * D;
     } else {
-        const int64_t slot = a.kv_loc[t];
         if (slot < 0) return;  // token without a cache slot: nothing of a K head is kept
         const int64_t row = (slot * a.hk + (h - a.hq)) * D;
         dst = static_cast<F *>(a.k_cache) + row;              // used when the cache has the activation type
@@ -967,15 +982,8 @@ __global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
 #pragma unroll
     for (int k = 0; k < PPL; ++k) {
         if (!live[k]) continue;
-        const int f = lane + 64 * k;  // rotary frequency of this pair
-        int64_t pos = p0;
-        if constexpr (AXES == 3) {
-            const bool on1 = (a.axis1[f >> 5] >> (f & 31)) & 1u, on2 = (a.axis2[f >> 5] >> (f & 31)) & 1u;
-            pos = on2 ? p2 : (on1 ? p1 : p0);
-        }
-        const F c = table[pos * D + f], s = table[pos * D + HALF + f];
-        const F n1 = w[i1[k]] * (x1[k] * rstd), n2 = w[i2[k]] * (x2[k] * rstd);
-        const F o1 = n1 * c - n2 * s, o2 = n2 * c + n1 * s;
+        const F n1 = w1[k] * (x1[k] * rstd), n2 = w2[k] * (x2[k] * rstd);
+        const F o1 = n1 * c[k] - n2 * s[k], o2 = n2 * c[k] + n1 * s[k];
         if (SETKV && KVFP8 && !is_q) {
             dst8[i1[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym((float)(o1 / (F)a.k_scale), kE4M3Max), 0.f, 0.f, 0.f);
             dst8[i2[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym((float)(o2 / (F)a.k_scale), kE4M3Max), 0.f, 0.f, 0.f);

@@ -172,7 +172,8 @@ int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *residual_in, 
 
 /*
  * The launch shape gpuk_add_rmsnorm_quant picks for a batch: lanes per token row (= workgroup size; one workgroup
- * per row) and 16-byte chunks per lane (0: rows too long for registers, swept three times).  For reports.
+ * per row) and chunks per lane (8 elements of a 16-bit type, 4 of fp32 / fp64; 0: rows too long for registers, swept
+ * three times).  For reports.
  */
 int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidden, int dtype, int *lanes_per_row,
                                         int *chunks_per_lane);

@@ -258,8 +258,12 @@ def test_launch_shape_report():
     assert capi.add_rmsnorm_quant_launch_shape(1, 4096) == (256, 2)
     lanes, chunks = capi.add_rmsnorm_quant_launch_shape(4, 65600 * 2)    # rows that do not stay in registers
     assert chunks == 0 and lanes % 64 == 0
-    lanes, chunks = capi.add_rmsnorm_quant_launch_shape(128, 1024, torch.float32)
-    assert chunks == 0 and lanes == 256
+    # fp32 / fp64: chunks of 4 elements, kept in registers up to 4 x 1024 of them
+    assert capi.add_rmsnorm_quant_launch_shape(128, 1024, torch.float32) == (128, 2)
+    assert capi.add_rmsnorm_quant_launch_shape(128, 1024, torch.float64) == (256, 1)
+    assert capi.add_rmsnorm_quant_launch_shape(128, 8192, torch.float64) == (1024, 2)
+    assert capi.add_rmsnorm_quant_launch_shape(128, 12288, torch.float32) == (768, 4)
+    assert capi.add_rmsnorm_quant_launch_shape(128, 16388, torch.float32) == (1024, 0)
     L = capi.lib()
     import ctypes as C
     a, b = C.c_int(0), C.c_int(0)

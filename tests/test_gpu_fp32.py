@@ -30,7 +30,7 @@ def close32(got, want, what):
 
 
 @pytest.mark.parametrize("dtype", WIDE)
-@pytest.mark.parametrize("tokens,hidden", [(33, 1024), (5, 8), (3, 16384), (64, 7168)])
+@pytest.mark.parametrize("tokens,hidden", [(33, 1024), (5, 8), (3, 16384), (64, 7168), (2, 20480), (7, 9000)])
 @pytest.mark.parametrize("quant", [0, 1, 3])
 def test_add_rmsnorm_quant_fp32(device, tokens, hidden, quant, dtype):
     from gpuk_amd import capi
