@@ -886,46 +886,62 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
 
 // ---------------------------------------------------------------------------------------------------------------
 // fp32 and fp64 activations: the reference dispatches them through the same templates (AT_DISPATCH_FLOATING_TYPES_AND2,
-// src/ops/fused_rope.cpp:27-30, :108-111).  A compatibility path, not a tuned one: one wave per (token, head), lane l
-// owns rotation pairs l, l+64, ...; with a KV cache the V heads get waves of their own that copy or quantise.
-// Rounding to the activation type F is the identity, so the oracle's sequence is plain arithmetic in F with every
-// product rounded before the add, around an fp32 variance and rstd (torch promotes x * rstd to F); an fp8 cache
-// takes float(o / F(scale)).
+// src/ops/fused_rope.cpp:27-30, :108-111).  The layout of the 16-bit kernel with chunks of 4 elements: a head is D/8
+// lanes, a lane owns the chunks at elements 4*sub and D/2 + 4*sub of its head (NeoX: x1 and x2 of frequencies
+// 4*sub .. 4*sub+3; GPT-J: the pairs of frequencies 2*sub, 2*sub+1 and D/4 + 2*sub, D/4 + 2*sub+1), a wave takes 512/D
+// consecutive Q/K heads of a token; with a KV cache further waves of the token copy or quantise its V row, 128 chunks
+// each.  Rounding to the activation type F is the identity, so the oracle's sequence is plain arithmetic in F with
+// every product rounded before the add, around an fp32 variance and rstd (torch promotes x * rstd to F); an fp8
+// cache takes float(o / F(scale)).
+constexpr int kWideChunksPerValueUnit = 128;
+template <int D> constexpr int wide_heads_per_wave() { return 512 / D; }
+
 template <typename F, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 __global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
-    constexpr int HALF = D / 2;
-    constexpr int PPL = (HALF + 63) / 64;  // pairs per lane
+    typedef F V4 __attribute__((ext_vector_type(4), aligned(16)));
+    constexpr int HALF = D / 2, LPH = D / 8, HPW = wide_heads_per_wave<D>();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t unit = blockIdx.x * (blockDim.x >> 6) + wave;
     if (unit >= a.total_units) return;
-    const int lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & 63, sub = lane % LPH, hl = lane / LPH;
     const uint32_t t = a.upt_magic ? __umulhi(unit, a.upt_magic) : unit;
-    const int h = (int)(unit - t * a.units_per_token);  // head index inside the token's qkv row
+    const int u = (int)(unit - t * a.units_per_token);  // unit inside the token
     const int heads_qk = a.hq + a.hk, heads_all = heads_qk + a.hv;
-    const F *src = static_cast<const F *>(a.qkv_in) + ((int64_t)t * heads_all + h) * D;
+    const int qk_units = (heads_qk + HPW - 1) / HPW;
+    const F *token_row = static_cast<const F *>(a.qkv_in) + (int64_t)t * heads_all * D;
 
-    if (h >= heads_qk) {  // a V head: only reached with a KV cache
+    if (u >= qk_units) {  // a share of the token's V row: only reached with a KV cache
         if constexpr (SETKV) {
             const int64_t slot = a.kv_loc[t];
             if (slot < 0) return;  // token without a cache slot
-            const int64_t row = (slot * a.hv + (h - heads_qk)) * D;
-            for (int e = lane; e < D; e += 64) {
-                const F v = src[e];
+            const int v_chunks = a.hv * (D / 4);
+#pragma unroll
+            for (int k = 0; k < kWideChunksPerValueUnit / 64; ++k) {
+                const int chunk = (u - qk_units) * kWideChunksPerValueUnit + 64 * k + lane;
+                if (chunk >= v_chunks) continue;
+                const V4 v = *reinterpret_cast<const V4 *>(token_row + (int64_t)heads_qk * D + 4 * chunk);
+                const int64_t off = slot * a.hv * D + 4 * (int64_t)chunk;
                 if constexpr (KVFP8) {
-                    static_cast<uint8_t *>(a.v_cache)[row + e] =
-                        (uint8_t)cvt4_e4m3fn(clamp_sym((float)(v / (F)a.v_scale), kE4M3Max), 0.f, 0.f, 0.f);
+                    const V4 q = v / (F)a.v_scale;
+                    *reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(a.v_cache) + off) =
+                        cvt4_e4m3fn(clamp_sym((float)q[0], kE4M3Max), clamp_sym((float)q[1], kE4M3Max),
+                                    clamp_sym((float)q[2], kE4M3Max), clamp_sym((float)q[3], kE4M3Max));
                 } else {
-                    static_cast<F *>(a.v_cache)[row + e] = v;
+                    *reinterpret_cast<V4 *>(static_cast<F *>(a.v_cache) + off) = v;
                 }
             }
         }
         return;
     }
 
-    const bool is_q = h < a.hq;
-    const F *w = static_cast<const F *>(is_q ? a.qw : a.kw);
-    // every load of the wave is issued before the first use: positions and slot (wave-uniform), then x, weights and
-    // the cos/sin values, whose rows depend on the positions
+    const int head_raw = u * HPW + hl;
+    const bool active = head_raw < heads_qk;
+    const int head = active ? head_raw : heads_qk - 1;  // idle lanes of a token's last unit repeat its last head
+    const bool is_q = head < a.hq;
+    const int e0 = 4 * sub, e1 = HALF + 4 * sub;
+
+    // every load of the wave is issued before the first use: positions and slot (wave-uniform), then x, the weights
+    // and the cos/sin values, whose rows depend on the positions
     const F *table = static_cast<const F *>(a.cos_sin);
     const int64_t p0 = a.positions[(int64_t)t * a.ps_token];
     int64_t p1 = p0, p2 = p0;
@@ -935,61 +951,87 @@ __global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
     }
     int64_t slot = 0;
     if constexpr (SETKV) slot = a.kv_loc[t];
-    F x1[PPL], x2[PPL], w1[PPL], w2[PPL], c[PPL], s[PPL];
-    int i1[PPL], i2[PPL];
-    bool live[PPL];
+    const F *src = token_row + (int64_t)head * D;
+    const V4 xa = *reinterpret_cast<const V4 *>(src + e0), xb = *reinterpret_cast<const V4 *>(src + e1);
+    const void *qw = a.qw, *kw = a.kw;
+    if constexpr (AXES == 3) asm("" : "+s"(qw), "+s"(kw));  // a select between kernel arguments: see RopeUnit::issue_loads
+    const F *w = static_cast<const F *>(is_q ? qw : kw);
+    const V4 wa = *reinterpret_cast<const V4 *>(w + e0), wb = *reinterpret_cast<const V4 *>(w + e1);
+    // the lane's four rotary frequencies, in the order the chunks' elements use them
+    int freq[4];
 #pragma unroll
-    for (int k = 0; k < PPL; ++k) {
-        const int f = lane + 64 * k;  // rotary frequency of this pair
-        live[k] = f < HALF;
-        const int fc = live[k] ? f : 0;
-        i1[k] = NEOX ? fc : 2 * fc;
-        i2[k] = NEOX ? fc + HALF : 2 * fc + 1;
-        x1[k] = live[k] ? src[i1[k]] : (F)0;
-        x2[k] = live[k] ? src[i2[k]] : (F)0;
-        w1[k] = w[i1[k]];
-        w2[k] = w[i2[k]];
-        int64_t pos = p0;
-        if constexpr (AXES == 3) {
-            const bool on1 = (a.axis1[fc >> 5] >> (fc & 31)) & 1u, on2 = (a.axis2[fc >> 5] >> (fc & 31)) & 1u;
-            pos = on2 ? p2 : (on1 ? p1 : p0);
+    for (int j = 0; j < 4; ++j) freq[j] = NEOX ? 4 * sub + j : (j < 2 ? 2 * sub + j : D / 4 + 2 * sub + (j - 2));
+    V4 c, s;
+    if (AXES == 1 || (p0 == p1 && p1 == p2)) {  // wave-uniform: one row, whole pieces of it
+        const F *row = table + p0 * D;
+        if constexpr (NEOX) {
+            c = *reinterpret_cast<const V4 *>(row + freq[0]);
+            s = *reinterpret_cast<const V4 *>(row + HALF + freq[0]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                c[j] = row[freq[j]];
+                s[j] = row[HALF + freq[j]];
+            }
         }
-        c[k] = table[pos * D + fc];
-        s[k] = table[pos * D + HALF + fc];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int f = freq[j];
+            const bool on1 = (bitmap_word<D>(a.axis1, f) >> (f & 31)) & 1u, on2 = (bitmap_word<D>(a.axis2, f) >> (f & 31)) & 1u;
+            const int64_t pos = on2 ? p2 : (on1 ? p1 : p0);
+            c[j] = table[pos * D + f];
+            s[j] = table[pos * D + HALF + f];
+        }
     }
+
     float ss = 0.f;
 #pragma unroll
-    for (int k = 0; k < PPL; ++k) {
-        const float f1 = (float)x1[k], f2 = (float)x2[k];
-        ss = __builtin_fmaf(f1, f1, ss);
-        ss = __builtin_fmaf(f2, f2, ss);
+    for (int j = 0; j < 4; ++j) {
+        const float fa = (float)xa[j], fb = (float)xb[j];
+        ss = __builtin_fmaf(fa, fa, ss);
+        ss = __builtin_fmaf(fb, fb, ss);
     }
-    ss = wave_allreduce<SumOp>(ss);
+    ss = group_allreduce<SumOp, LPH < 16 ? LPH : 16>(ss);
+    if constexpr (LPH == 32) ss += __shfl_xor(ss, 16);
     const F rstd = (F)(1.0f / sqrtf(ss * (1.0f / D) + a.eps));
 
-    F *dst;
-    uint8_t *dst8 = nullptr;
+    const V4 na = wa * (xa * rstd), nb = wb * (xb * rstd);
+    V4 oa, ob;
+    if constexpr (NEOX) {
+        oa = na * c - nb * s;
+        ob = nb * c + na * s;
+    } else {
+        oa = V4{na[0] * c[0] - na[1] * s[0], na[1] * c[0] + na[0] * s[0], na[2] * c[1] - na[3] * s[1], na[3] * c[1] + na[2] * s[1]};
+        ob = V4{nb[0] * c[2] - nb[1] * s[2], nb[1] * c[2] + nb[0] * s[2], nb[2] * c[3] - nb[3] * s[3], nb[3] * c[3] + nb[2] * s[3]};
+    }
+    if (!active) return;
+    // rotated rows are stored past the L2 (as the 16-bit kernel does from a few MB per call on; smaller calls are
+    // bound by their launch either way)
     if constexpr (!SETKV) {
-        dst = static_cast<F *>(a.qkv_out) + ((int64_t)t * heads_all + h) * D;
+        F *dst = static_cast<F *>(a.qkv_out) + ((int64_t)t * heads_all + head) * D;
+        __builtin_nontemporal_store(oa, reinterpret_cast<V4 *>(dst + e0));
+        __builtin_nontemporal_store(ob, reinterpret_cast<V4 *>(dst + e1));
     } else if (is_q) {
-        dst = static_cast<F *>(a.q_out) + ((int64_t)t * a.hq + h) * D;
+        F *dst = static_cast<F *>(a.q_out) + ((int64_t)t * a.hq + head) * D;
+        __builtin_nontemporal_store(oa, reinterpret_cast<V4 *>(dst + e0));
+        __builtin_nontemporal_store(ob, reinterpret_cast<V4 *>(dst + e1));
     } else {
         if (slot < 0) return;  // token without a cache slot: nothing of a K head is kept
-        const int64_t row = (slot * a.hk + (h - a.hq)) * D;
-        dst = static_cast<F *>(a.k_cache) + row;              // used when the cache has the activation type
-        dst8 = static_cast<uint8_t *>(a.k_cache) + row;       // used when it is fp8
-    }
-#pragma unroll
-    for (int k = 0; k < PPL; ++k) {
-        if (!live[k]) continue;
-        const F n1 = w1[k] * (x1[k] * rstd), n2 = w2[k] * (x2[k] * rstd);
-        const F o1 = n1 * c[k] - n2 * s[k], o2 = n2 * c[k] + n1 * s[k];
-        if (SETKV && KVFP8 && !is_q) {
-            dst8[i1[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym((float)(o1 / (F)a.k_scale), kE4M3Max), 0.f, 0.f, 0.f);
-            dst8[i2[k]] = (uint8_t)cvt4_e4m3fn(clamp_sym((float)(o2 / (F)a.k_scale), kE4M3Max), 0.f, 0.f, 0.f);
+        const int64_t row = (slot * a.hk + (head - a.hq)) * D;
+        if constexpr (KVFP8) {
+            const V4 qa = oa / (F)a.k_scale, qb = ob / (F)a.k_scale;
+            uint8_t *dst = static_cast<uint8_t *>(a.k_cache) + row;
+            *reinterpret_cast<uint32_t *>(dst + e0) =
+                cvt4_e4m3fn(clamp_sym((float)qa[0], kE4M3Max), clamp_sym((float)qa[1], kE4M3Max),
+                            clamp_sym((float)qa[2], kE4M3Max), clamp_sym((float)qa[3], kE4M3Max));
+            *reinterpret_cast<uint32_t *>(dst + e1) =
+                cvt4_e4m3fn(clamp_sym((float)qb[0], kE4M3Max), clamp_sym((float)qb[1], kE4M3Max),
+                            clamp_sym((float)qb[2], kE4M3Max), clamp_sym((float)qb[3], kE4M3Max));
         } else {
-            dst[i1[k]] = o1;
-            dst[i2[k]] = o2;
+            F *dst = static_cast<F *>(a.k_cache) + row;
+            __builtin_nontemporal_store(oa, reinterpret_cast<V4 *>(dst + e0));
+            __builtin_nontemporal_store(ob, reinterpret_cast<V4 *>(dst + e1));
         }
     }
 }
@@ -1320,6 +1362,12 @@ void build_axis_bitmaps(const int64_t *section, bool interleaved, int half, uint
     }
 }
 
+// Waves per token of the fp32 / fp64 kernel: 512/D consecutive Q/K heads each, then 128 chunks of the V row each.
+int64_t wide_units_per_token(int64_t hq, int64_t hk, int64_t hv, int64_t D, bool set_kv) {
+    const int64_t hpw = 512 / D, v_chunks = set_kv ? hv * (D / 4) : 0;
+    return (hq + hk + hpw - 1) / hpw + (v_chunks + kWideChunksPerValueUnit - 1) / kWideChunksPerValueUnit;
+}
+
 int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *kw, const void *cos_sin,
                 const int64_t *positions, int64_t ps_axis, int64_t ps_token, int n_axes, int64_t T, int64_t hq,
                 int64_t hk, int64_t hv, int64_t D, int neox, const int64_t *section, int interleaved, float eps,
@@ -1359,7 +1407,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
     int64_t upt = (hq + hk + hpw - 1) / hpw;
     if (hq + hk == 0) return GPUK_ERR_UNSUPPORTED;  // a qkv row without Q and K heads has nothing to rotate
     const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
-    if (wide) upt = hq + hk + (set_kv ? hv : 0);  // the fp32 / fp64 path: one wave per head
+    if (wide) upt = wide_units_per_token(hq, hk, hv, D, set_kv);
     // mulhi(unit, ceil(2^32/upt)) equals unit / upt while unit * upt < 2^32
     if (upt * T >= 0x7fffffffLL || upt * T * upt >= (1LL << 32)) return GPUK_ERR_UNSUPPORTED;
     a.qkv_in = qkv_in;
@@ -1398,7 +1446,7 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
     if (!walking || !workgroups || !lanes || !streamed) return GPUK_ERR_INVALID_ARG;
     const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
     const int64_t hpw = 64 / (D / 16);
-    const int64_t upt = wide ? hq + hk + (set_kv ? hv : 0) : (hq + hk + hpw - 1) / hpw;
+    const int64_t upt = wide ? wide_units_per_token(hq, hk, hv, D, set_kv) : (hq + hk + hpw - 1) / hpw;
     if (upt * T >= 0x7fffffffLL || upt * T * upt >= (1LL << 32)) return GPUK_ERR_UNSUPPORTED;
     RopeArgs a{};
     a.total_units = (uint32_t)(upt * T);

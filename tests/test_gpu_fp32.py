@@ -110,28 +110,29 @@ def test_rope_inplace_fp32(device, head_size, neox, mrope, interleaved, dtype):
 @pytest.mark.parametrize("dtype", WIDE)
 @pytest.mark.parametrize("fp8_cache", [False, True])
 @pytest.mark.parametrize("mrope", [False, True])
-def test_rope_set_kv_fp32(device, fp8_cache, mrope, dtype):
+@pytest.mark.parametrize("D,neox", [(128, True), (128, False), (64, True), (256, False)])
+def test_rope_set_kv_fp32(device, fp8_cache, mrope, dtype, D, neox):
     import gpuk_amd as gpuk
 
     kv_dtype = torch.float8_e4m3fn if fp8_cache else dtype
-    print(f"case {dtype} rope set_kv cache={kv_dtype} mrope={mrope}", flush=True)
-    T, hq, hk, hv, D = 45, 8, 2, 2, 128
-    inp = rope_case(T, hq, hk, hv, D, True, 77, mrope, False, kv_dtype, dtype)
+    print(f"case {dtype} rope set_kv cache={kv_dtype} mrope={mrope} D={D} neox={neox}", flush=True)
+    T, hq, hk, hv = 45, 7, 2, 3     # a last Q/K wave with idle lanes; at D=256 a second, partly filled V wave
+    inp = rope_case(T, hq, hk, hv, D, neox, 77 + D, mrope, False, kv_dtype, dtype)
     inp.kv_loc[3] = -1            # a padding token: q_out row written, K and V rows dropped
     qkv, qw, kw, cs, pos, loc = (t.to(device) for t in (inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, inp.kv_loc))
     k0, v0 = inp.new_cache()
     kc, vc = k0.to(device), v0.to(device)
     q_out = torch.empty((T, hq, D), dtype=dtype, device=device)
     if mrope:
-        gpuk.fused_mrope_3d_rms_set_kv(qkv, qw, kw, cs, pos, T, hq, hk, hv, D, True, inp.mrope_section, False, inp.eps,
+        gpuk.fused_mrope_3d_rms_set_kv(qkv, qw, kw, cs, pos, T, hq, hk, hv, D, neox, inp.mrope_section, False, inp.eps,
                                        q_out, kc, vc, loc, inp.k_scale, inp.v_scale)
     else:
-        gpuk.fused_rope_rms_set_kv(qkv, qw, kw, cs, pos, T, hq, hk, hv, D, True, inp.eps, q_out, kc, vc, loc,
+        gpuk.fused_rope_rms_set_kv(qkv, qw, kw, cs, pos, T, hq, hk, hv, D, neox, inp.eps, q_out, kc, vc, loc,
                                    inp.k_scale, inp.v_scale)
     torch.cuda.synchronize()
     q_ref = torch.empty((T, hq, D), dtype=dtype)
     k_ref, v_ref = k0.clone(), v0.clone()
-    O.rope_rms_set_kv_ref(inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, T, hq, hk, hv, D, True, inp.eps, q_ref,
+    O.rope_rms_set_kv_ref(inp.qkv, inp.qw, inp.kw, inp.cos_sin, inp.positions, T, hq, hk, hv, D, neox, inp.eps, q_ref,
                           k_ref, v_ref, inp.kv_loc, inp.k_scale, inp.v_scale, inp.mrope_section, False)
     close32(q_out, q_ref, "q_out")
     kc, vc = kc.cpu(), vc.cpu()
