@@ -243,15 +243,10 @@ struct RopeUnit {
         st.head = min(head_raw, heads_qk - 1);
         st.is_q = st.head < a.hq;
         const uint16_t *src = st.token_in + (int64_t)st.head * D;
-        // streamed when the results go elsewhere; in place the same lines are written a moment later, and keeping
-        // them in L2 measured 2 % faster
-        if constexpr (SETKV) {
-            st.xa = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c0(sub)));
-            st.xb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c1(sub)));
-        } else {
-            st.xa = *reinterpret_cast<const u32x4 *>(src + c0(sub));
-            st.xb = *reinterpret_cast<const u32x4 *>(src + c1(sub));
-        }
+        // streamed, in place too (the lines are written a moment later, but past the L2: keeping them there cost 2-17 %
+        // from 512 tokens on once the stores were streamed)
+        st.xa = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c0(sub)));
+        st.xb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c1(sub)));
 
         // this wave's share of the token's V row: chunk u*64 + lane (and further strides of units_per_token*64)
         if constexpr (SETKV) {
@@ -1207,10 +1202,12 @@ int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allo
 //                      chip's 1024 SIMDs, so its run time moves in steps of ceil(waves / 1024) waves per SIMD (one
 //                      token per wave, 40 heads: 9.2 us at 1024 tokens, 12.1 at 2048, 15.4 at 3072, 19.0 at 4096,
 //                      and 14.5-14.8 anywhere from 2400 to 2800) while the other kernel's grows with the tokens.
-//                      Against the other kernel with streaming stores it is ahead only with one position axis, a
-//                      16-bit cache, head size 128 and one token per wave on a grid whose last step is full with three
-//                      or four waves on every SIMD (40 heads: 18.45 against 18.9 us at 4096 tokens, 14.9 against 15.1
-//                      at 3072; in place 15.9 against 16.6).  Elsewhere the other kernel is level or ahead: 33.6
+//                      Against the other kernel with streaming stores it is ahead only when writing a 16-bit cache,
+//                      with one position axis, head size 128 and one token per wave on a grid whose last step is full
+//                      with three or four waves on every SIMD (40 heads: 18.45 against 18.9 us at 4096 tokens, 14.9
+//                      against 15.1 at 3072).  In place the other kernel, its loads streamed as well, is ahead at
+//                      every size (40 heads: 12.4 against 14.2 us at 3000 tokens, 15.8 against 20.0 at 4096, 28.4
+//                      against 32.7 at 8192).  Elsewhere it is level or ahead too: 33.6
 //                      against 35.8 us at 8192 x 40 heads, 64.8 against 69.0 at 16384, 28.0 against 31.5 at 4096 x 72
 //                      heads with an fp8 cache, 65.6 against 70.7 at 8192 x 40 heads of 256, with three position axes
 //                      27.0 against 27.7 at 8192 x 32 heads and 50.7 against 51.9 at 16384 (16.5 both at 4096 with
@@ -1245,7 +1242,7 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     const uint32_t simds = 4 * kComputeUnits;
     const uint32_t waves_per_simd = (p.walk_waves + simds - 1) / simds;  // of the fullest SIMD
     const bool last_step_full = waves_per_simd >= 3 && 100 * (uint64_t)p.walk_waves >= 95 * (uint64_t)waves_per_simd * simds;
-    const bool slots_filled = last_step_full && axes == 1 && !kv_fp8 && D == 128 && tokens_per_wave == 1;
+    const bool slots_filled = last_step_full && set_kv && axes == 1 && !kv_fp8 && D == 128 && tokens_per_wave == 1;
     p.walk = v_fits && strides_fit &&
              (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits && slots_filled));
     // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows

@@ -278,6 +278,8 @@ def test_rope_launch_shape_report():
     from gpuk_amd import capi
     # 4096 tokens x (32, 8, 8) heads of 128: one wave per token fills every SIMD four times -> the walking kernel
     assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128) == (True, 1024, 256, False)
+    # in place the kernel with one wave per group of heads is ahead at every size
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, set_kv=False) == (False, 5120, 256, True)
     # three position axes, or an fp8 cache: one wave per group of 8 heads, four waves a workgroup, streamed stores
     assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3) == (False, 8192, 256, True)
     assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (False, 5120, 256, True)
