@@ -914,7 +914,7 @@ __global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
             for (int k = 0; k < kWideChunksPerValueUnit / 64; ++k) {
                 const int chunk = (u - qk_units) * kWideChunksPerValueUnit + 64 * k + lane;
                 if (chunk >= v_chunks) continue;
-                const V4 v = *reinterpret_cast<const V4 *>(token_row + (int64_t)heads_qk * D + 4 * chunk);
+                const V4 v = __builtin_nontemporal_load(reinterpret_cast<const V4 *>(token_row + (int64_t)heads_qk * D + 4 * chunk));
                 const int64_t off = slot * a.hv * D + 4 * (int64_t)chunk;
                 if constexpr (KVFP8) {
                     const V4 q = v / (F)a.v_scale;
@@ -947,7 +947,8 @@ __global__ void __launch_bounds__(256) rope_rms_wide_kernel(const RopeArgs a) {
     int64_t slot = 0;
     if constexpr (SETKV) slot = a.kv_loc[t];
     const F *src = token_row + (int64_t)head * D;
-    const V4 xa = *reinterpret_cast<const V4 *>(src + e0), xb = *reinterpret_cast<const V4 *>(src + e1);
+    const V4 xa = __builtin_nontemporal_load(reinterpret_cast<const V4 *>(src + e0));
+    const V4 xb = __builtin_nontemporal_load(reinterpret_cast<const V4 *>(src + e1));
     const void *qw = a.qw, *kw = a.kw;
     if constexpr (AXES == 3) asm("" : "+s"(qw), "+s"(kw));  // a select between kernel arguments: see RopeUnit::issue_loads
     const F *w = static_cast<const F *>(is_q ? qw : kw);
