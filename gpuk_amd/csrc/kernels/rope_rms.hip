@@ -1458,7 +1458,7 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
         *walking = 0;
         *workgroups = (int)((a.total_units + 3) / 4);
         *lanes = 256;
-        *streamed = 0;
+        *streamed = 1;  // the fp32 / fp64 kernel always stores its rotated rows past the L2
         return GPUK_OK;
     }
     const RopePlan p = plan_rope(a, (int)D, n_axes, set_kv, set_kv && kv_dtype == GPUK_KV_E4M3FN);

@@ -287,9 +287,9 @@ def test_rope_launch_shape_report():
     assert capi.rope_rms_launch_shape(16, 28, 4, 4, 128) == (False, 16, 256, False)
     assert capi.rope_rms_launch_shape(16, 40, 8, 8, 128, kv_fp8=True) == (False, 96, 64, False)
     # fp32 activations: a wave per 512/D Q/K heads, and per 512 elements of the V row when a cache is written
-    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32) == (False, 5, 256, False)
-    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32, set_kv=False) == (False, 3, 256, False)
-    assert capi.rope_rms_launch_shape(4, 7, 2, 3, 256, dtype=torch.float64) == (False, 7, 256, False)
+    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32) == (False, 5, 256, True)
+    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32, set_kv=False) == (False, 3, 256, True)
+    assert capi.rope_rms_launch_shape(4, 7, 2, 3, 256, dtype=torch.float64) == (False, 7, 256, True)
     import ctypes as C
     L = capi.lib()
     o = [C.c_int(0) for _ in range(4)]
