@@ -296,8 +296,11 @@ def main():
         def copy_same_bytes_us(nbytes):
             """The plain copy kernel moving as many bytes as a call of a fused kernel moves (half in, half out)."""
             half = (nbytes // 2 + 15) // 16 * 16
+            if half > nb:   # a shape given on the command line whose calls move more than the copy buffers hold
+                return None
             room = nb - half
-            offs = [(k * half) % room // 256 * 256 for k in range(3)]   # three windows of the 512 MiB buffers
+            # three windows of the 512 MiB buffers (the same window three times when only one fits)
+            offs = [((k * half) % room // 256 * 256) if room > 0 else 0 for k in range(3)]
             return round(event_time_ms(lambda i=0: capi.copy_bytes(dst[offs[i % 3]:], src[offs[i % 3]:], half), 100) * 1e3, 2)
 
         # the fused kernel's own memory traffic without its arithmetic (same launch shape, mapping, streaming accesses

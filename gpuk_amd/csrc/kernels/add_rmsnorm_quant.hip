@@ -248,8 +248,8 @@ add_rmsnorm_quant_traffic_only(const u32x4 *x, const u32x4 *residual_in, u32x4 *
 // three sweeps over the row, re-reading what this same lane wrote to residual_out (L2-resident).
 template <typename T, int QUANT>
 __global__ void __launch_bounds__(kMaxThreads)
-add_rmsnorm_quant_long_rows(const u32x4 *__restrict__ x, const u32x4 *__restrict__ residual_in,
-                            const u32x4 *__restrict__ gamma, u32x4 *residual_out, void *__restrict__ norm_out,
+add_rmsnorm_quant_long_rows(const u32x4 *x, const u32x4 *residual_in,  // either may be residual_out: no __restrict__
+                            const u32x4 *__restrict__ gamma, u32x4 *residual_out, void *norm_out,
                             float *__restrict__ scale_io, int chunks_per_row, float hidden_f, float eps,
                             float fp8_max) {
     using P = Pack16<T>;
@@ -335,8 +335,8 @@ using wide4 = F __attribute__((ext_vector_type(4)));
 
 template <typename F, int QUANT, int CPL>
 __global__ void __launch_bounds__(kMaxThreads)
-add_rmsnorm_quant_wide_rows(const wide4<F> *__restrict__ x, const wide4<F> *__restrict__ residual_in,
-                            const wide4<F> *__restrict__ gamma, wide4<F> *residual_out, void *__restrict__ norm_out,
+add_rmsnorm_quant_wide_rows(const wide4<F> *x, const wide4<F> *residual_in,  // either may be residual_out
+                            const wide4<F> *__restrict__ gamma, wide4<F> *residual_out, void *norm_out,
                             float *__restrict__ scale_io, int chunks_per_row, float hidden_f, float eps, float fp8_max) {
     __shared__ float s_sum[kReduceSlots];
     __shared__ float s_max[kReduceSlots];
@@ -610,9 +610,9 @@ extern "C" int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidde
                                                    int *chunks_per_lane) {
     using namespace gpuk;
     if (tokens <= 0 || hidden <= 0 || !lanes_per_row || !chunks_per_lane) return GPUK_ERR_INVALID_ARG;
+    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32 && dtype != GPUK_DTYPE_F64) return GPUK_ERR_UNSUPPORTED;
     const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
-    const int elems = wide ? 4 : 8;
-    if (hidden % elems != 0) return GPUK_ERR_UNSUPPORTED;
+    if (hidden % 8 != 0) return GPUK_ERR_UNSUPPORTED;  // the rule of gpuk_add_rmsnorm_quant, for every dtype
     if (wide) {  // the fp32 / fp64 kernel: 4-element chunks, 0 = rows swept three times
         pick_wide_shape((int)(hidden / 4), dtype == GPUK_DTYPE_F64, lanes_per_row, chunks_per_lane);
         return GPUK_OK;

@@ -190,7 +190,9 @@ __device__ __forceinline__ void norm_rotate(const u32x4 &xa, const u32x4 &xb, co
 template <int OFFSET>
 __device__ __forceinline__ void store_pair(void *p, const u32x4 &a, const u32x4 &b, bool nt) {
     if (nt) {
-        asm volatile("global_store_dwordx4 %0, %1, off nt\n\tglobal_store_dwordx4 %0, %2, off offset:%3 nt" ::"v"(p), "v"(a), "v"(b), "n"(OFFSET) : "memory");
+        // the trailing s_nop: a store wider than 64 bits needs one wait state before its data registers may be
+        // overwritten, and the compiler's hazard pass does not look inside an asm statement
+        asm volatile("global_store_dwordx4 %0, %1, off nt\n\tglobal_store_dwordx4 %0, %2, off offset:%3 nt\n\ts_nop 0" ::"v"(p), "v"(a), "v"(b), "n"(OFFSET) : "memory");
     } else {
         *reinterpret_cast<u32x4 *>(p) = a;
         *reinterpret_cast<u32x4 *>(static_cast<char *>(p) + OFFSET) = b;
@@ -417,25 +419,29 @@ __device__ __forceinline__ const void *in_scalar_registers(const void *p) {
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo);
 }
+// The transfers are self-sufficient about hardware hazards, because the compiler's hazard pass does not look inside
+// an asm statement: `s_nop 4` gives the five wait states a vector memory instruction needs after a v_readfirstlane
+// wrote the scalar registers it takes its base from (and the one it needs after M0 was written), and M0 is named as
+// clobbered.
 template <bool NT>
 __device__ __forceinline__ void lds_fill16(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
     if constexpr (NT) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc", "m0");
     } else {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc", "m0");
     }
 }
 // the same for lanes 0-31 only: 512 bytes of LDS
 __device__ __forceinline__ void lds_fill16_lanes32(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
     uint64_t saved_exec;
-    asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc");
+    asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc", "m0");
 }
 // ... with a full address per lane (the lanes may read from different rows)
 __device__ __forceinline__ void lds_fill16_lanes32_gather(uint32_t lds_byte_offset, const void *lane_address) {
     uint64_t saved_exec;
-    asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_address) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_address) : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void wait_fills() {  // until at most N vector memory instructions are outstanding
@@ -569,7 +575,7 @@ struct RopeWalk {
         // one transfer with per-lane addresses relative to qw: lanes 32-63 reach over to kw
         const int64_t k_minus_q = kw - qw;
         const uint32_t within = (16u * (lane & 31)) % (2u * D);
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(qw + (lane < 32 ? 0 : k_minus_q) + within) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(qw + (lane < 32 ? 0 : k_minus_q) + within) : "memory", "m0");
     }
     __device__ __forceinline__ void take_weights(const unsigned char *at) {
         u32x4 qa = *reinterpret_cast<const u32x4 *>(at + 16 * sub), qb = *reinterpret_cast<const u32x4 *>(at + D + 16 * sub);
@@ -866,8 +872,12 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
             w.template finish_unit<Walk::kK>(xa, xb, v, cur_v, stream_q);
             issued += slot_ok ? 2 : 0;
         } else {
+            // Lanes of both kinds, or Q lanes beside lanes past the last head.  Only stores that some lane takes part
+            // in are counted: with no lane active a store sequence may be branched over, and a count above what was
+            // issued would let a later wait return before its transfer has landed.
             w.template finish_unit<Walk::kMixed>(xa, xb, v, cur_v, stream_q);
-            issued += SETKV && slot_ok ? 4 : 2;  // in place one store sequence serves both kinds of lanes
+            const bool has_k_lane = (uint32_t)a.hq < min(h0 + (uint32_t)HPW, (uint32_t)heads_qk);
+            issued += SETKV && slot_ok && has_k_lane ? 4 : 2;  // in place one store sequence serves both kinds of lanes
         }
         if (SETKV && cur_v && slot_ok) issued += 1;
         cslot = cslot + 1 == (uint32_t)RING ? 0 : cslot + 1;
@@ -1442,6 +1452,7 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
     if (T <= 0 || hq < 0 || hk < 0 || hv < 0 || hq + hk == 0 || (n_axes != 1 && n_axes != 3)) return GPUK_ERR_INVALID_ARG;
     if (D != 64 && D != 128 && D != 256) return GPUK_ERR_UNSUPPORTED;
     if (!walking || !workgroups || !lanes || !streamed) return GPUK_ERR_INVALID_ARG;
+    if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32 && dtype != GPUK_DTYPE_F64) return GPUK_ERR_UNSUPPORTED;
     const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
     const int64_t hpw = 64 / (D / 16);
     const int64_t upt = wide ? wide_units_per_token(hq, hk, hv, D, set_kv) : (hq + hk + hpw - 1) / hpw;

@@ -263,13 +263,17 @@ def test_launch_shape_report():
     assert capi.add_rmsnorm_quant_launch_shape(128, 1024, torch.float64) == (256, 1)
     assert capi.add_rmsnorm_quant_launch_shape(128, 8192, torch.float64) == (1024, 2)
     assert capi.add_rmsnorm_quant_launch_shape(128, 12288, torch.float32) == (768, 4)
-    assert capi.add_rmsnorm_quant_launch_shape(128, 16388, torch.float32) == (1024, 0)
+    assert capi.add_rmsnorm_quant_launch_shape(128, 16392, torch.float32) == (1024, 0)
     L = capi.lib()
     import ctypes as C
     a, b = C.c_int(0), C.c_int(0)
     assert L.gpuk_add_rmsnorm_quant_launch_shape(0, 1024, 0, C.byref(a), C.byref(b)) == 1
     assert L.gpuk_add_rmsnorm_quant_launch_shape(4, 1027, 0, C.byref(a), C.byref(b)) == 2
     assert L.gpuk_add_rmsnorm_quant_launch_shape(4, 1024, 0, None, C.byref(b)) == 1
+    # the query refuses what the entry point refuses: rows that are no multiple of 8 elements (whatever the dtype),
+    # and a dtype value that names no format
+    assert L.gpuk_add_rmsnorm_quant_launch_shape(4, 16388, 2, C.byref(a), C.byref(b)) == 2
+    assert L.gpuk_add_rmsnorm_quant_launch_shape(4, 1024, 7, C.byref(a), C.byref(b)) == 2
 
 
 def test_rope_launch_shape_report():
@@ -298,3 +302,4 @@ def test_rope_launch_shape_report():
     assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 96, 1, 0, 1, 0, *refs) == 2
     assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 128, 2, 0, 1, 0, *refs) == 1
     assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 128, 1, 0, 1, 0, None, *refs[1:]) == 1
+    assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 128, 1, 9, 1, 0, *refs) == 2   # no such dtype

@@ -56,6 +56,36 @@ def test_add_rmsnorm_quant_fp32(device, tokens, hidden, quant, dtype):
             assert_scales_close(scale, scale_ref, "scales")
 
 
+@pytest.mark.parametrize("dtype", WIDE)
+@pytest.mark.parametrize("alias", ["residual_in", "x"])
+@pytest.mark.parametrize("quant", [0, 1, 3])
+def test_residual_out_may_alias_an_input_fp32(device, alias, quant, dtype):
+    """The in-place residual stream for fp32 / fp64 activations: residual_out is the same buffer as residual_in or x.
+    Rows kept in registers (1, 2 and 4 chunks per lane) and rows swept three times, where a lane reads back what it
+    stored (20480 elements), all give the results of separate buffers."""
+    from gpuk_amd import capi
+
+    for tokens, hidden in ((33, 1024), (9, 7168), (3, 16384), (4, 20480)):
+        print(f"case {dtype} alias={alias} quant={quant} {tokens}x{hidden}", flush=True)
+        inp = workloads.norm_quant_inputs(tokens, hidden, seed=hidden + quant, res_sigma=1.5, outlier_frac=0.01, dtype=dtype)
+        static = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
+        x, r, g = inp.x.to(device), inp.residual.to(device), inp.gamma.to(device)
+        norm = torch.empty((tokens, hidden), dtype=dtype if quant == 0 else torch.float8_e4m3fn, device=device)
+        scale = None if quant == 0 else (torch.full((tokens, 1), -1.0, device=device) if quant == 1
+                                         else static.to(device).float().reshape(1))
+        res = r if alias == "residual_in" else x
+        capi.add_rmsnorm_quant(x, r, g, res, norm, scale, inp.eps, quant)
+        torch.cuda.synchronize()
+        res_ref, norm_ref, scale_ref = O.add_rmsnorm_quant_ref(inp.x, inp.residual, inp.gamma, inp.eps, quant, static_scale=static)
+        assert_bits_equal(res.cpu().view(INT_OF[dtype]), res_ref.view(INT_OF[dtype]), "residual_out")
+        if quant == 0:
+            close32(norm, norm_ref, "norm_out")
+        else:
+            assert_codes_close(norm, norm_ref, "codes")
+            if quant == 1:
+                assert_scales_close(scale, scale_ref, "scales")
+
+
 def test_torch_op_accepts_fp32(device):
     import gpuk_amd as gpuk
 

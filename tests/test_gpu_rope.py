@@ -158,10 +158,12 @@ def test_mrope_set_kv_sweep(device, neox, interleaved, head_size, fp8):
     check_set_kv(inp, run_set_kv(inp, device), "[mrope set_kv]")
 
 
-@pytest.mark.parametrize("hq,hk,hv", [(32, 8, 8), (28, 4, 4), (64, 8, 8), (5, 3, 2), (1, 1, 1), (40, 40, 40)])
+@pytest.mark.parametrize("hq,hk,hv", [(32, 8, 8), (28, 4, 4), (64, 8, 8), (5, 3, 2), (1, 1, 1), (40, 40, 40),
+                                      (36, 0, 8), (13, 0, 3), (0, 13, 5), (0, 5, 2), (0, 16, 16)])
 @pytest.mark.parametrize("fp8", [True, False])
 def test_rope_set_kv_head_mixes(device, hq, hk, hv, fp8):
-    """GQA head mixes, including counts that do not fill a wave's group of heads."""
+    """GQA head mixes, including counts that do not fill a wave's group of heads and calls without K heads or without
+    Q heads (then the cache or q_out is an empty tensor)."""
     print(f"case set_kv heads={hq},{hk},{hv} fp8={fp8}", flush=True)
     inp = make(67, hq, 128, True, seed=hq * 100 + hk, fp8=fp8, hk=hk, hv=hv)
     check_set_kv(inp, run_set_kv(inp, device), f"[set_kv {hq},{hk},{hv}]")
@@ -213,6 +215,11 @@ WALK_CASES = [
     (23, (7, 2, 0), 128, True, False, False, False),      # no V heads
     (41, (28, 4, 4), 128, True, "aligned", False, False),  # sections on multiples of 8: the rows arrive merged
     (27, (6, 2, 2), 64, False, "aligned", False, True),   # the same with GPT-J pairs, head size 64, fp8 cache
+    (31, (36, 0, 8), 128, True, False, False, False),     # no K heads: the last unit holds Q lanes and idle lanes only
+    (31, (13, 0, 3), 128, False, False, False, True),     # the same with an fp8 cache, GPT-J pairs
+    (35, (21, 0, 5), 64, True, True, False, False),       # no K heads, 16 heads per unit, three position axes
+    (31, (0, 13, 5), 128, True, False, False, False),     # no Q heads
+    (29, (0, 5, 2), 128, False, True, True, True),        # no Q heads, fp8 cache, interleaved sections
 ]
 ALIGNED_SECTIONS = {64: [8, 16, 8], 128: [16, 24, 24], 256: [48, 40, 40]}
 
