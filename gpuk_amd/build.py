@@ -1,7 +1,10 @@
-"""In-tree build of the two shared libraries (run as `python -m gpuk_amd.build`).
+"""In-tree build of the shared libraries (run as `python -m gpuk_amd.build`).
 
   gpuk_amd/lib/libgpuk_amd.so : HIP kernels for gfx950 behind the C ABI of include/gpuk_amd.h (no torch)
   gpuk_amd/lib/libgpuk.so     : torch library `gpuk` (csrc/register.cpp + csrc/ops/*.cpp), links the former
+  gpuk_amd/lib/libgpuk_amd_stamps.so : the first, compiled with -DGPUK_STAMPS: a profiling build whose kernels
+                                record the shader clock at named phases (`python -m gpuk_amd.stamps`); `--stamps`
+                                builds only this one
 
 hipcc cross-compiles gfx950 code objects without a GPU, so this runs on a CPU-only builder; the
 built files travel with the tree.  The reference builds with CMake for either CUDA or HIP
@@ -29,6 +32,11 @@ DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fno-gp
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall"]
 
 KERNEL_SOURCES = ["kernels/add_rmsnorm_quant.hip", "kernels/rope_rms.hip", "kernels/calibration.hip", "kernels/capi.cpp"]
+# Kernel-argument preload: the first 14 dwords of a kernel's arguments are placed in scalar registers when a wave is
+# launched, so its first loads do not wait for a fetch of the argument block (the norm-quant kernel orders its
+# and the rope kernels order their arguments for this).
+EXTRA_FLAGS = {"kernels/add_rmsnorm_quant.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"],
+               "kernels/rope_rms.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"]}
 OP_SOURCES = ["register.cpp", "ops/allreduce_rms.cpp", "ops/fused_rope.cpp"]
 
 
@@ -48,17 +56,23 @@ def _compile(args):
     return obj
 
 
-def build_kernels(jobs: int = 4) -> str:
+def build_kernels(jobs: int = 4, stamps: bool = False) -> str:
+    """libgpuk_amd.so, or with stamps=True libgpuk_amd_stamps.so: the same sources compiled with -DGPUK_STAMPS, in
+    which the kernels record the shader clock at named phases (read by `python -m gpuk_amd.stamps`)."""
     os.makedirs(LIB, exist_ok=True)
     work = []
     for s in KERNEL_SOURCES:
         flags = list(DEVICE_FLAGS)
         if s.endswith(".cpp"):
             flags = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include"]
-        work.append((s, os.path.join(OBJ, s.replace("/", "_") + ".o"), flags))
+        else:
+            flags += EXTRA_FLAGS.get(s, [])
+            if stamps:
+                flags.append("-DGPUK_STAMPS")
+        work.append((s, os.path.join(OBJ, ("stamps_" if stamps else "") + s.replace("/", "_") + ".o"), flags))
     with ThreadPoolExecutor(jobs) as ex:
         objs = list(ex.map(_compile, work))
-    out = os.path.join(LIB, "libgpuk_amd.so")
+    out = os.path.join(LIB, "libgpuk_amd_stamps.so" if stamps else "libgpuk_amd.so")
     _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", out] + objs)
     return out
 
@@ -93,8 +107,14 @@ def build_all(verbose: bool = True) -> None:
     b = build_torch_library()
     if verbose:
         print("built", b)
+    c = build_kernels(stamps=True)
+    if verbose:
+        print("built", c)
 
 
 if __name__ == "__main__":
-    build_all()
+    if "--stamps" in sys.argv[1:]:
+        print("built", build_kernels(stamps=True))
+    else:
+        build_all()
     sys.exit(0)

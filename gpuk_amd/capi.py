@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "lib
 EXPORTS = ("gpuk_status_string", "gpuk_abi_version", "gpuk_add_rmsnorm_quant", "gpuk_rope_rms",
            "gpuk_rope_rms_set_kv", "gpuk_rope_rms_2way", "gpuk_copy_bytes", "gpuk_increment_floats", "gpuk_set_tuning",
            "gpuk_add_rmsnorm_quant_traffic_only", "gpuk_add_rmsnorm_quant_launch_shape",
-           "gpuk_rope_rms_launch_shape")
+           "gpuk_rope_rms_launch_shape", "gpuk_read_bytes", "gpuk_fill_bytes", "gpuk_empty_grid")
 
 DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2, torch.float64: 3}
 QUANT_NONE, QUANT_FP8_DYNAMIC, QUANT_FP8_E4M3FNUZ, QUANT_FP8_STATIC = 0, 1, 2, 3
@@ -30,6 +30,12 @@ class GpukError(RuntimeError):
 
 
 _lib = None
+
+
+def use_library(path: str) -> None:
+    """Bind this module to another build of the C ABI (the profiling build libgpuk_amd_stamps.so) from here on."""
+    global _lib, _LIB_PATH
+    _LIB_PATH, _lib = path, None
 
 
 def lib():
@@ -65,6 +71,12 @@ def lib():
         L.gpuk_rope_rms_launch_shape.argtypes = [C.c_int64] * 5 + [C.c_int] * 4 + [C.POINTER(C.c_int)] * 4
         L.gpuk_copy_bytes.restype = C.c_int
         L.gpuk_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
+        L.gpuk_read_bytes.restype = C.c_int
+        L.gpuk_read_bytes.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]
+        L.gpuk_fill_bytes.restype = C.c_int
+        L.gpuk_fill_bytes.argtypes = [C.c_void_p, C.c_int64, C.c_uint32, C.c_void_p]
+        L.gpuk_empty_grid.restype = C.c_int
+        L.gpuk_empty_grid.argtypes = [C.c_int64, C.c_int, C.c_int, C.c_void_p]
         _lib = L
     return _lib
 
@@ -167,6 +179,24 @@ def copy_bytes(dst, src, nbytes: int, stream=None) -> None:
     rc = lib().gpuk_copy_bytes(_ptr(dst), _ptr(src), nbytes, _stream(stream))
     if rc:
         raise GpukError(rc, "gpuk_copy_bytes")
+
+
+def read_bytes(src, nbytes: int, sink, stream=None) -> None:
+    rc = lib().gpuk_read_bytes(_ptr(src), nbytes, _ptr(sink), _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_read_bytes")
+
+
+def fill_bytes(dst, nbytes: int, seed: int = 1, stream=None) -> None:
+    rc = lib().gpuk_fill_bytes(_ptr(dst), nbytes, seed & 0xFFFFFFFF, _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_fill_bytes")
+
+
+def empty_grid(workgroups: int, lanes: int, lds_bytes: int = 0, stream=None) -> None:
+    rc = lib().gpuk_empty_grid(workgroups, lanes, lds_bytes, _stream(stream))
+    if rc:
+        raise GpukError(rc, "gpuk_empty_grid")
 
 
 def rope_rms_2way(q0, k0, q1, k1, w_q0, w_k0, w_q1, w_k1, cos_sin0, cos_sin1, batch_size, T0, T1, Hq, Hk, D,

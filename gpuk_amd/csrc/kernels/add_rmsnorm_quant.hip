@@ -61,18 +61,25 @@ __device__ __forceinline__ float div_by_rcp_finite(float a, float b, float rcp) 
     return __builtin_fmaf(-e, rcp, q);
 }
 
-template <typename T, int NCHUNK, int QUANT>
+// EXACT: lanes x NCHUNK equals the chunks of a row, so every lane owns NCHUNK live chunks and nothing is masked
+// (true for every power-of-two row and for 7168 elements; it removes a sixth of the kernel's instructions, which is
+// what a decode-sized batch waits for: with at most one row per compute unit the run time is the row's arithmetic).
+template <typename T, int NCHUNK, int QUANT, bool EXACT>
 __global__ void __launch_bounds__(kMaxThreads)
-add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
-                       const u32x4 *__restrict__ gamma, u32x4 *residual_out, void *norm_out,
-                       float *__restrict__ scale_io, int tokens, int chunks_per_row, float hidden_f, float rcp_hidden,
-                       int hidden_pow2, float eps, float fp8_max, int group_shift, int remap_end) {
+add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_row, int remap_end, int group_shift,
+                       int nthreads, const u32x4 *__restrict__ gamma, u32x4 *residual_out, void *norm_out,
+                       float *__restrict__ scale_io, float hidden_f, float rcp_hidden, int hidden_pow2, float eps,
+                       float fp8_max, float rcp_fp8_max) {
+    // The arguments are ordered by when a wave needs them: the first fourteen dwords (up to norm_out) are handed to
+    // the wave in scalar registers at launch (-amdgpu-kernarg-preload-count), so the loads of the row are issued
+    // without a round trip for the argument block; nthreads is the workgroup size, passed so that it need not be
+    // fetched from the dispatch packet either.
     using P = Pack16<T>;
     __shared__ float s_sum[kReduceSlots];
     __shared__ float s_max[kReduceSlots];
+    GPUK_STAMPS_BEGIN();  // profiling build only; slots: see kNormQuantStampNames
 
     const int tid = threadIdx.x;
-    const int nthreads = blockDim.x;
     const int num_waves = nthreads >> 6;
     // Workgroup ids are handed to the 8 XCDs round-robin.  Below remap_end the rows are dealt out in runs of
     // 2^group_shift consecutive rows per XCD instead of one row each (which rows run concurrently stays the same;
@@ -91,7 +98,7 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
 #pragma unroll
     for (int i = 0; i < NCHUNK; ++i) {
         const int c = i * nthreads + tid;
-        live[i] = c < chunks_per_row;
+        live[i] = EXACT || c < chunks_per_row;
         if (live[i]) {
             xv[i] = load_stream(x + row_base + c);
             rv[i] = load_stream(residual_in + row_base + c);
@@ -105,6 +112,8 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
         const int c = i * nthreads + tid;
         gv[i] = live[i] ? gamma[c] : u32x4{0, 0, 0, 0};
     }
+    GPUK_STAMP(1);          // every load issued
+    GPUK_STAMP_DRAINED(2);  // ... and landed
 
     // ---- phase 1: res = rT(x + r), stored once; sum of squares of the *rounded* residual.  Waves in this phase
     // are given issue priority over the arithmetic of phases 2-3 so that their residual stores leave early (+0.4 %).
@@ -122,14 +131,22 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
         if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
     }
     float sumsq[1] = {ss0 + ss1};
+    GPUK_STAMP(3);  // residual stored, the lane's squares summed
     block_allreduce<SumOp, 1>(sumsq, s_sum, num_waves);
     __builtin_amdgcn_s_setprio(0);
+    GPUK_STAMP(4);  // sum of squares of the row known to every wave
 
     // ---- phase 2: n2 = rT(gamma * rT(res * rstd)); row amax for the dynamic scale.
     // mean = sumsq / H as an exact IEEE quotient: a multiplication when H is a power of two (exact, and rounded like
     // the quotient when the result is subnormal), a division otherwise
-    const float mean = hidden_pow2 ? sumsq[0] * rcp_hidden : sumsq[0] / hidden_f;
-    const float rstd = 1.0f / sqrtf(mean + eps);
+    // Elsewhere the quotient by multiply and two fused multiply-adds (exact on the guarded range, see div_by_rcp) and
+    // the short square root and reciprocal: every wave of the row walks this dependent chain before it can go on.
+    float mean;
+    if (hidden_pow2) mean = sumsq[0] * rcp_hidden;
+    else if (__builtin_expect(__builtin_amdgcn_ballot_w64(!in_mid_range(sumsq[0])) == 0, 1)) mean = div_by_rcp_finite(sumsq[0], hidden_f, rcp_hidden);
+    else mean = sumsq[0] / hidden_f;
+    const float rstd = rsqrt_two_roundings(mean + eps);
+    GPUK_STAMP(5);  // rstd
     if constexpr (QUANT == GPUK_QUANT_NONE) {
         u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base;
 #pragma unroll
@@ -142,6 +159,9 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
             }
             if (live[i]) store_stream(out + i * nthreads + tid, xv[i]);
         }
+        GPUK_STAMP(9);
+        GPUK_STAMP_DRAINED(10);
+        GPUK_STAMPS_WRITE(blockIdx.x * num_waves + (tid >> 6));
         return;
     } else {
         // the normed row stays in fp32 registers, every value already rounded to the 16-bit type.
@@ -165,10 +185,16 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
             }
         }
         float scale;
+        GPUK_STAMP(6);  // row normed, the lane's maximum known
         if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
             float amax[1] = {any_nan ? __builtin_nanf("") : __builtin_fmaxf(m0, m1)};
             block_allreduce<MaxOp, 1>(amax, s_max, num_waves);
-            scale = amax[0] == 0.f ? 1.f : amax[0] / fp8_max;
+            GPUK_STAMP(7);  // row maximum known to every wave
+            // rcp_fp8_max is RN(1 / fp8_max) for the two maxima the quotient was checked for (448, 240), else 0
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(in_mid_range(amax[0]) && rcp_fp8_max != 0.f)) == 0, 1))
+                scale = div_by_rcp_finite(amax[0], fp8_max, rcp_fp8_max);
+            else
+                scale = amax[0] == 0.f ? 1.f : amax[0] / fp8_max;
             if (tid == 0) scale_io[row] = scale;
         } else {
             scale = scale_io[0];
@@ -181,7 +207,10 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
         constexpr bool kDynamic = QUANT == GPUK_QUANT_FP8_DYNAMIC;
         u32x2 *out = reinterpret_cast<u32x2 *>(norm_out) + row_base;
         if (__builtin_expect(scale_in_fast_range(scale), 1)) {
-            const float rcp = 1.0f / scale;
+            float rcp;
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(mantissa_all_ones(scale)) == 0, 1)) rcp = rcp_rn_mid_range(scale);
+            else rcp = 1.0f / scale;
+            GPUK_STAMP(8);  // scale and its reciprocal
 #pragma unroll
             for (int i = 0; i < NCHUNK; ++i) {
                 float q[8];
@@ -203,6 +232,9 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in,
                 if (live[i]) store_stream(out + i * nthreads + tid, codes);
             }
         }
+        GPUK_STAMP(9);           // codes stored (issued)
+        GPUK_STAMP_DRAINED(10);  // every store of the wave acknowledged
+        GPUK_STAMPS_WRITE(blockIdx.x * num_waves + (tid >> 6));
     }
 }
 
@@ -478,16 +510,23 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
     }
     const float rcp_hidden = 1.0f / hf;
     const int hidden_pow2 = (hidden & (hidden - 1)) == 0;
-    const int tok = (int)tokens;
+    const float rcp_fp8_max = (fp8_max == 448.0f || fp8_max == 240.0f) ? 1.0f / fp8_max : 0.0f;
     // Runs of 64 rows per XCD: measured +1.1 % for 16 KiB rows (8192 rows); neutral or 1-10 % slower for every other
     // row size tried (2, 3, 4, 8, 10, 14, 32 KiB) and for fewer rows, hence the narrow rule.
     const int64_t row_bytes = hidden * 2;
     int group_shift = row_bytes == 16384 && tokens >= 1024 ? 6 : 0;
     if (g_row_group_shift >= 0) group_shift = g_row_group_shift;
     const int remap_end = group_shift > 0 ? (int)((tokens >> (3 + group_shift)) << (3 + group_shift)) : 0;
-#define GPUK_LAUNCH_NQ(N)                                                                                         \
-    add_rmsnorm_quant_rows<T, N, QUANT><<<grid, threads, 0, stream>>>(xs, rs, gs, ro, norm_out, scale, tok, chunks, hf, \
-                                                                      rcp_hidden, hidden_pow2, eps, fp8_max, group_shift, remap_end)
+    const bool exact = (int64_t)threads * nchunk == chunks;
+#define GPUK_LAUNCH_NQ(N)                                                                                              \
+    do {                                                                                                               \
+        if (exact)                                                                                                     \
+            add_rmsnorm_quant_rows<T, N, QUANT, true><<<grid, threads, 0, stream>>>(                                   \
+                xs, rs, chunks, remap_end, group_shift, threads, gs, ro, norm_out, scale, hf, rcp_hidden, hidden_pow2, eps, fp8_max, rcp_fp8_max); \
+        else                                                                                                           \
+            add_rmsnorm_quant_rows<T, N, QUANT, false><<<grid, threads, 0, stream>>>(                                  \
+                xs, rs, chunks, remap_end, group_shift, threads, gs, ro, norm_out, scale, hf, rcp_hidden, hidden_pow2, eps, fp8_max, rcp_fp8_max); \
+    } while (0)
     switch (nchunk) {
         case 1: GPUK_LAUNCH_NQ(1); break;
         case 2: GPUK_LAUNCH_NQ(2); break;
@@ -577,6 +616,9 @@ void set_norm_quant_tuning(int key, int value) {
 }
 
 }  // namespace gpuk
+
+// profiling build: where the kernels of this file write their phase stamps
+GPUK_STAMPS_SETTER(gpuk_stamps_set_norm_quant)
 
 extern "C" int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *residual_in, void *residual_out,
                                                    void *codes, float *scale, int64_t tokens, int64_t hidden,

@@ -186,4 +186,103 @@ __device__ __forceinline__ float div_by_rcp(float a, float b, float rcp) {
     return __builtin_amdgcn_div_fixupf(__builtin_fmaf(e, rcp, q), b, a);
 }
 
+// ---- Correctly rounded square root and reciprocal by short sequences.  The compiler's expansions of sqrtf() and of
+// 1.0f / x are correct for every operand and pay for it with rescaling and fix-up steps (about 20 and 11 dependent
+// instructions); on operands in the middle of the exponent range those steps do nothing.  These start from
+// v_sqrt_f32 / v_rcp_f32 (1 ULP) and correct the result; oracle/gpuk_oracle.c holds the same sequences and
+// tests/test_oracle_norm_quant.py runs them over every mantissa from every first guess within one ULP: they return the
+// correctly rounded value except the reciprocal of a number whose mantissa bits are all ones, which callers exclude.
+__device__ __forceinline__ float sqrt_rn_mid_range(float v) {  // v in [2^-95, 2^97)
+    const float s = __builtin_amdgcn_sqrtf(v);
+    const float dn = __builtin_bit_cast(float, __builtin_bit_cast(int32_t, s) - 1);
+    const float up = __builtin_bit_cast(float, __builtin_bit_cast(int32_t, s) + 1);
+    const float r_dn = __builtin_fmaf(-dn, s, v), r_up = __builtin_fmaf(-up, s, v);
+    const float t = r_dn <= 0.0f ? dn : s;
+    return r_up > 0.0f ? up : t;
+}
+__device__ __forceinline__ float rcp_rn_mid_range(float s) {  // s in [2^-60, 2^60], mantissa not all ones
+    float y = __builtin_amdgcn_rcpf(s);
+    y = __builtin_fmaf(__builtin_fmaf(-s, y, 1.0f), y, y);
+    return __builtin_fmaf(__builtin_fmaf(-s, y, 1.0f), y, y);
+}
+__device__ __forceinline__ bool in_mid_range(float v) {  // [2^-60, 2^60): one subtraction and one unsigned compare
+    return __builtin_bit_cast(uint32_t, v) - 0x21800000u < 0x3c000000u;
+}
+__device__ __forceinline__ bool mantissa_all_ones(float v) {
+    return (__builtin_bit_cast(uint32_t, v) & 0x7fffffu) == 0x7fffffu;
+}
+// 1 / sqrt(v), both steps correctly rounded, as `1.0f / sqrtf(v)`.  The choice between the short and the general
+// sequence is made for the whole wave, so the common case has no divergent branch.
+__device__ __forceinline__ float rsqrt_two_roundings(float v) {
+    const float s = sqrt_rn_mid_range(v);
+    const bool ok = in_mid_range(v) && !mantissa_all_ones(s);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!ok) == 0, 1)) return rcp_rn_mid_range(s);
+    return 1.0f / sqrtf(v);
+}
+
+// ---- Phase stamps (profiling build only: -DGPUK_STAMPS, `python -m gpuk_amd.build --stamps`).  A wave reads the
+// shader clock at named points of a kernel and keeps the readings in scalar registers; at its end lane 0 writes them,
+// with the 100 MHz wall clock at entry and exit and the wave's place on the chip, to a host-provided buffer of
+// kStampSlots 64-bit words per wave.  In the product build every macro below expands to nothing.
+constexpr int kStampSlots = 16;
+#ifdef GPUK_STAMPS
+static __device__ uint64_t *g_stamp_buffer;   // one copy per translation unit, set by that unit's gpuk_stamps_* entry
+static __device__ uint32_t g_stamp_waves;     // waves the buffer has room for
+struct Stamps {
+    uint64_t t[kStampSlots - 3];
+    uint64_t wall0;
+    __device__ __forceinline__ static uint64_t cycles() {
+        uint64_t v;
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v)::"memory");
+        __builtin_amdgcn_sched_barrier(0);
+        return v;
+    }
+    __device__ __forceinline__ static uint64_t wall() {
+        uint64_t v;
+        asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v)::"memory");
+        return v;
+    }
+    __device__ __forceinline__ void begin() {
+#pragma unroll
+        for (int i = 0; i < kStampSlots - 3; ++i) t[i] = 0;
+        wall0 = wall();
+        t[0] = cycles();
+    }
+    // every vector memory operation of the wave has completed: loads have landed, stores are acknowledged
+    __device__ __forceinline__ static void drain() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+    __device__ __forceinline__ void write(uint32_t wave_index) const {
+        const uint64_t wall1 = wall();
+        uint32_t hw_id, xcc_id;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_id));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
+        if (g_stamp_buffer && wave_index < g_stamp_waves && (threadIdx.x & 63) == 0) {
+            uint64_t *out = g_stamp_buffer + (uint64_t)wave_index * kStampSlots;
+#pragma unroll
+            for (int i = 0; i < kStampSlots - 3; ++i) out[i] = t[i];
+            out[kStampSlots - 3] = wall0;
+            out[kStampSlots - 2] = wall1;
+            out[kStampSlots - 1] = ((uint64_t)(xcc_id & 0xf) << 32) | hw_id;
+        }
+    }
+};
+#define GPUK_STAMPS_BEGIN() gpuk::Stamps stamps_; stamps_.begin()
+#define GPUK_STAMP(slot) (stamps_.t[slot] = gpuk::Stamps::cycles())
+#define GPUK_STAMP_DRAINED(slot) (gpuk::Stamps::drain(), stamps_.t[slot] = gpuk::Stamps::cycles())
+#define GPUK_STAMPS_WRITE(wave_index) stamps_.write(wave_index)
+#define GPUK_STAMPS_SETTER(name)                                                                                     \
+    extern "C" int name(void *buffer, uint32_t waves) {                                                                \
+        uint64_t *b = static_cast<uint64_t *>(buffer);                                                                 \
+        if (hipMemcpyToSymbol(HIP_SYMBOL(gpuk::g_stamp_buffer), &b, sizeof(b)) != hipSuccess) return GPUK_ERR_INTERNAL; \
+        if (hipMemcpyToSymbol(HIP_SYMBOL(gpuk::g_stamp_waves), &waves, sizeof(waves)) != hipSuccess) return GPUK_ERR_INTERNAL; \
+        return GPUK_OK;                                                                                                \
+    }
+#else
+#define GPUK_STAMPS_BEGIN() ((void)0)
+#define GPUK_STAMP(slot) ((void)0)
+#define GPUK_STAMP_DRAINED(slot) ((void)0)
+#define GPUK_STAMPS_WRITE(wave_index) ((void)0)
+#define GPUK_STAMPS_SETTER(name)
+#endif
+
 }  // namespace gpuk

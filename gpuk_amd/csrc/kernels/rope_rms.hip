@@ -38,17 +38,17 @@ constexpr float kE4M3Max = 448.0f;
 
 struct RopeArgs {
     const void *qkv_in;
-    void *qkv_out;  // == qkv_in for the in-place form, unused for set_kv
-    const void *qw, *kw, *cos_sin;
     const int64_t *positions;
-    int64_t ps_axis, ps_token;
-    void *q_out, *k_cache, *v_cache;
     const int64_t *kv_loc;
     // one wave per unit = (token, group of heads); units_per_token = ceil((hq + hk) / heads per wave)
     uint32_t total_units, units_per_token;
     uint32_t upt_magic;  // ceil(2^32 / units_per_token), or 0 when units_per_token is 1: unit / units_per_token is
                          // mulhi(unit, magic) for every unit the host admits
     int hq, hk, hv;
+    int64_t ps_axis, ps_token;
+    void *qkv_out;  // == qkv_in for the in-place form, unused for set_kv
+    const void *qw, *kw, *cos_sin;
+    void *q_out, *k_cache, *v_cache;
     float eps, k_scale, v_scale;
     // mRoPE: bit f of axis1 / axis2 set when rotary frequency f takes its position from axis 1 / 2
     uint32_t axis1[4], axis2[4];
@@ -147,7 +147,7 @@ __device__ __forceinline__ void norm_rotate(const u32x4 &xa, const u32x4 &xb, co
         ss1 = P::add_squares(xb[j], ss1);
     }
     const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
-    const float rstd = 1.0f / sqrtf(sumsq * (1.0f / D) + eps);  // D is a power of two: the product is exact
+    const float rstd = rsqrt_two_roundings(sumsq * (1.0f / D) + eps);  // D is a power of two: the product is exact
 
     // normed values stay in fp32 registers, each already rounded to the 16-bit type
     float na[8], nb[8];
@@ -252,21 +252,21 @@ struct RopeUnit {
 
         // this wave's share of the token's V row: chunk u*64 + lane (and further strides of units_per_token*64)
         if constexpr (SETKV) {
-            st.slot = a.kv_loc[st.t];
             const int v_first = st.u * 64 + lane;
             if (v_first < a.hv * (D / 8))
                 st.vchunk = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(st.token_in + (int64_t)heads_qk * D + 8 * v_first));
         }
-
-        const uint16_t *wsrc = static_cast<const uint16_t *>(st.is_q ? qw : kw);
-        st.wa = *reinterpret_cast<const u32x4 *>(wsrc + c0(sub));
-        st.wb = *reinterpret_cast<const u32x4 *>(wsrc + c1(sub));
-
         st.p0 = a.positions[(int64_t)st.t * a.ps_token];
         if constexpr (AXES == 3) {
             st.p1 = a.positions[a.ps_axis + (int64_t)st.t * a.ps_token];
             st.p2 = a.positions[2 * a.ps_axis + (int64_t)st.t * a.ps_token];
         }
+        // so far nothing needed more than the kernel's leading parameters, which a wave finds in its registers; the
+        // slot and the weights are reached through pointers of the argument block
+        if constexpr (SETKV) st.slot = a.kv_loc[st.t];
+        const uint16_t *wsrc = static_cast<const uint16_t *>(st.is_q ? qw : kw);
+        st.wa = *reinterpret_cast<const u32x4 *>(wsrc + c0(sub));
+        st.wb = *reinterpret_cast<const u32x4 *>(wsrc + c1(sub));
     }
 
     // The cos/sin loads, whose addresses wait for the positions.
@@ -375,20 +375,46 @@ struct RopeUnit {
     }
 };
 
+// What a wave needs to ask for its activations and its position(s) comes as 14 dwords of leading scalar parameters,
+// which are handed to the wave in scalar registers at launch (-amdgpu-kernarg-preload-count=14): those requests
+// leave without a round trip for the argument block, which under load costs a wave of this kernel a third of its
+// life; the block (weights, table, outputs, slots) is fetched beside the position, and everything that depends on
+// either is asked for one round trip after entry.  hv_and_waves: hv in bits 0-23, log2 of the waves per workgroup above.
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
-__global__ void __launch_bounds__(512) rope_rms_kernel(const RopeArgs a) {
+__global__ void __launch_bounds__(512)
+rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_units, uint32_t units_per_token,
+                uint32_t upt_magic, int hq, int hk, uint32_t hv_and_waves, int64_t ps_token, int64_t ps_axis,
+                const RopeArgs rest) {
     using Unit = RopeUnit<T, D, NEOX, AXES, SETKV, KVFP8>;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t unit = blockIdx.x * (blockDim.x >> 6) + wave;
-    if (unit >= a.total_units) return;
+    const uint32_t unit = (blockIdx.x << (hv_and_waves >> 24)) + wave;
+    if (unit >= total_units) return;
+    RopeArgs a = rest;  // the fields that came ahead replace their copies in the block
+    a.qkv_in = qkv_in;
+    a.positions = positions;
+    a.total_units = total_units;
+    a.units_per_token = units_per_token;
+    a.upt_magic = upt_magic;
+    a.hq = hq;
+    a.hk = hk;
+    a.hv = (int)(hv_and_waves & 0xffffffu);
+    a.ps_token = ps_token;
+    a.ps_axis = ps_axis;
+    GPUK_STAMPS_BEGIN();  // profiling build only; slots: see kRopeUnitStampNames
     const int lane = threadIdx.x & 63;
     UnitState st;
     Unit::issue_loads(a, unit, lane, st);
+    GPUK_STAMP(1);  // activations, weights, position and slot requested
     Unit::issue_table_loads(a, lane, st);
+    GPUK_STAMP(2);  // position known, cos/sin requested
     // Every load of the wave is in flight before the first use of any of them: without this fence the scheduler
     // moves arithmetic above later loads and the wave pays several memory round trips in a row.
     __builtin_amdgcn_sched_barrier(0);
+    GPUK_STAMP_DRAINED(3);  // everything landed
     Unit::finish(a, lane, st);
+    GPUK_STAMP(4);          // rows stored (issued)
+    GPUK_STAMP_DRAINED(5);  // ... and acknowledged
+    GPUK_STAMPS_WRITE(unit);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -422,7 +448,11 @@ __device__ __forceinline__ const void *in_scalar_registers(const void *p) {
 // The transfers are self-sufficient about hardware hazards, because the compiler's hazard pass does not look inside
 // an asm statement: `s_nop 4` gives the five wait states a vector memory instruction needs after a v_readfirstlane
 // wrote the scalar registers it takes its base from (and the one it needs after M0 was written), and M0 is named as
-// clobbered.
+// clobbered, so that the compiler never carries a value of its own in M0 across a transfer (it answers with a
+// warning that M0 is a reserved register, silenced below: reserved means it allocates nothing there, which is the
+// point).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 template <bool NT>
 __device__ __forceinline__ void lds_fill16(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
     if constexpr (NT) {
@@ -443,6 +473,7 @@ __device__ __forceinline__ void lds_fill16_lanes32_gather(uint32_t lds_byte_offs
     asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
                  : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_address) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 template <int N>
 __device__ __forceinline__ void wait_fills() {  // until at most N vector memory instructions are outstanding
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -480,7 +511,7 @@ __device__ __forceinline__ void norm_rotate_unpacked(const u32x4 &xa, const u32x
         ss1 = P::add_squares(xb[j], ss1);
     }
     const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
-    const float rstd = 1.0f / sqrtf(sumsq * (1.0f / D) + eps);
+    const float rstd = rsqrt_two_roundings(sumsq * (1.0f / D) + eps);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const float a0 = P::round(w[2 * j] * P::round(P::lo(xa[j]) * rstd));
@@ -570,6 +601,8 @@ struct RopeWalk {
         lds_fill16_lanes32_gather(dst, static_cast<const char *>(cos_sin) + pos * (2 * D) + 16 * piece);
     }
     // Both weight vectors -> 1 KiB at `dst`: q weights in the first 512 bytes, k weights in the second
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
     __device__ __forceinline__ void fill_weights(uint32_t dst) const {
         const char *qw = static_cast<const char *>(a.qw), *kw = static_cast<const char *>(a.kw);
         // one transfer with per-lane addresses relative to qw: lanes 32-63 reach over to kw
@@ -577,6 +610,7 @@ struct RopeWalk {
         const uint32_t within = (16u * (lane & 31)) % (2u * D);
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(qw + (lane < 32 ? 0 : k_minus_q) + within) : "memory", "m0");
     }
+#pragma clang diagnostic pop
     __device__ __forceinline__ void take_weights(const unsigned char *at) {
         u32x4 qa = *reinterpret_cast<const u32x4 *>(at + 16 * sub), qb = *reinterpret_cast<const u32x4 *>(at + D + 16 * sub);
         u32x4 ka = *reinterpret_cast<const u32x4 *>(at + 512 + 16 * sub), kb = *reinterpret_cast<const u32x4 *>(at + 512 + D + 16 * sub);
@@ -728,6 +762,7 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t first = blockIdx.x * kWalkWaves + wave;
     if (first >= n_waves) return;  // the host keeps the number of waves <= the number of tokens
+    GPUK_STAMPS_BEGIN();  // profiling build only; slots: see kRopeWalkStampNames
     Walk w(a, threadIdx.x & 63, qkv_in, cos_sin, heads_qk, heads_all, hv);
     w.t = first;
     w.u = 0;
@@ -818,8 +853,11 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
     fill_table(p0, p1, p2);
 #pragma unroll
     for (int i = 1; i < RING; ++i) stage_next();
+    GPUK_STAMP(1);  // every transfer of the prologue issued (the first position has arrived)
     wait_fills_upto(__builtin_amdgcn_readfirstlane(issued - weights_mark));
     w.take_weights(reinterpret_cast<const unsigned char *>(&s_w[wave][0]));
+    GPUK_STAMP(2);  // norm weights arrived and unpacked
+    [[maybe_unused]] uint32_t units_done = 0;
 
     // One step: wait for the current unit's transfers (and, at a token's first unit, for its table rows), move it to
     // registers, refill what that freed (next token's rows, next unit's V share, the unit RING ahead), finish the unit.
@@ -831,6 +869,9 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
         if (cur_v) newest = max(newest, v_mark);
         if (token_start) newest = max(newest, rows_mark);
         wait_fills_upto(__builtin_amdgcn_readfirstlane(issued - newest));  // uniform anyway; keeps the switch scalar
+#ifdef GPUK_STAMPS
+        if (units_done == 0) GPUK_STAMP(3);  // the first unit and its table row arrived
+#endif
         const u32x4 *stage = &s_stage[wave][0][0] + cslot * 128;
         u32x4 xa = stage[w.lane], xb = stage[64 + w.lane], v = u32x4{0, 0, 0, 0};
         in_registers(xa);
@@ -880,6 +921,13 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
             issued += SETKV && slot_ok && has_k_lane ? 4 : 2;  // in place one store sequence serves both kinds of lanes
         }
         if (SETKV && cur_v && slot_ok) issued += 1;
+#ifdef GPUK_STAMPS
+        // the stores of the wave's first eight units issued: slots 4 .. 11 (a select chain: the slot is not a constant)
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (units_done == (uint32_t)k) GPUK_STAMP(4 + k);
+        ++units_done;
+#endif
         cslot = cslot + 1 == (uint32_t)RING ? 0 : cslot + 1;
         if (++w.u == upt) {
             w.u = 0;
@@ -887,6 +935,8 @@ rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__res
             if (w.t >= tokens) break;
         }
     }
+    GPUK_STAMP_DRAINED(12);  // every store of the wave acknowledged
+    GPUK_STAMPS_WRITE(first);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1201,6 +1251,7 @@ int g_walk_waves = 0;       // waves the walking grid may hold at once (0 = buil
 int g_walk_stream = 0;      // streaming stores of the walking kernel: 0 = built-in rule, 1 = never, 2 = always
 int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
 
+
 // Which kernel and which stores, measured on MI355X (32/8/8, 28/4/4 and 64/8/8 heads, head sizes 64-256, random slots):
 //   streaming stores : in the one-wave-per-unit kernel, q_out / K rows / in-place rows written past the L2 are ahead
 //                      from about 10 MB per call on (64+8 heads, fp8 cache: 5.9 against 7.0 us at 512 tokens, 16.0
@@ -1291,7 +1342,10 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
             a.hq + a.hk + a.hv, (int)a.ps_token, (int)a.ps_axis, a.hv, b);
         return hip_status(hipGetLastError());
     }
-    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<p.blocks, p.threads, 0, stream>>>(b);
+    const uint32_t log2_waves = p.threads == 64 ? 0u : p.threads == 128 ? 1u : p.threads == 256 ? 2u : 3u;
+    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<p.blocks, p.threads, 0, stream>>>(
+        a.qkv_in, a.positions, a.total_units, a.units_per_token, a.upt_magic, a.hq, a.hk,
+        (uint32_t)a.hv | (log2_waves << 24), a.ps_token, a.ps_axis, b);
     return hip_status(hipGetLastError());
 }
 
@@ -1491,6 +1545,9 @@ void set_rope_tuning(int key, int value) {
 }
 
 }  // namespace gpuk
+
+// profiling build: where the kernels of this file write their phase stamps
+GPUK_STAMPS_SETTER(gpuk_stamps_set_rope)
 
 extern "C" int gpuk_rope_rms_launch_shape(int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k,
                                           int64_t num_heads_v, int64_t head_size, int n_axes, int dtype, int set_kv,

@@ -160,6 +160,25 @@ int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1, const voi
 int gpuk_copy_bytes(void *dst, const void *src, int64_t nbytes, void *stream);
 
 /*
+ * Roofline calibration, one direction at a time: gpuk_read_bytes reads src[0..nbytes) with the copy kernel's tiles
+ * and streaming loads and writes nothing (`sink`, 4 bytes of device memory, receives a word only if a fold of the
+ * data hits one fixed value); gpuk_fill_bytes writes dst[0..nbytes) with the copy kernel's streaming stores and
+ * reads nothing.  A kernel that reads R and writes W bytes is priced against R / read-only rate + W / write-only
+ * rate.  nbytes a multiple of 16, pointers 16-byte aligned.  The reference's micro-benchmark measures the copy
+ * only (test/cpp/global_memory_bandwidth.cpp:95-114); these are its two halves.
+ */
+int gpuk_read_bytes(const void *src, int64_t nbytes, void *sink, void *stream);
+int gpuk_fill_bytes(void *dst, int64_t nbytes, uint32_t seed, void *stream);
+
+/*
+ * Launch-cost calibration for a grid shape: `workgroups` workgroups of `lanes_per_workgroup` lanes (a multiple of 64,
+ * at most 1024) with `lds_bytes` of dynamic LDS each (at most 65536) that return at once.  Its duration is what
+ * launching, placing and draining that grid costs before any byte moves.  Same purpose as the reference's
+ * test/cpp/test_small_kernel.cpp:98-178, for a full-size grid.
+ */
+int gpuk_empty_grid(int64_t workgroups, int lanes_per_workgroup, int lds_bytes, void *stream);
+
+/*
  * Roofline calibration: the memory traffic of gpuk_add_rmsnorm_quant (16-bit activations, fp8 output, per-token
  * scale) without its arithmetic: same launch shape, lane-to-data mapping, streaming loads and stores and barriers;
  * residual_out receives x ^ residual_in, codes a fold of it, scale 1.0 per token.  Its duration is the ceiling of the

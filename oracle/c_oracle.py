@@ -58,6 +58,9 @@ def lib():
             [C.c_void_p] * 10 + [C.c_int64] * 6 + [C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p])
         L.gpuk_oracle_count_div_rcp_mismatch.restype = C.c_int64
         L.gpuk_oracle_count_div_rcp_mismatch.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        for name in ("gpuk_oracle_count_short_sqrt_mismatch", "gpuk_oracle_count_short_rcp_mismatch"):
+            getattr(L, name).restype = C.c_int64
+            getattr(L, name).argtypes = [C.c_uint32, C.c_int64, C.c_int]
         _lib = L
     return _lib
 
@@ -126,3 +129,13 @@ def count_div_rcp_mismatch(a: torch.Tensor, b: torch.Tensor) -> int:
     """a, b: fp32 CPU tensors of equal length; see gpuk_oracle_count_div_rcp_mismatch."""
     assert a.dtype == torch.float32 and b.dtype == torch.float32 and a.numel() == b.numel()
     return lib().gpuk_oracle_count_div_rcp_mismatch(_p(a.contiguous()), _p(b.contiguous()), a.numel())
+
+
+def count_short_sqrt_mismatch(first_bits: int, n: int, first_guess_ulp: int) -> int:
+    """See gpuk_oracle_count_short_sqrt_mismatch: fp32 bit patterns first_bits .. first_bits + n - 1."""
+    return lib().gpuk_oracle_count_short_sqrt_mismatch(first_bits, n, first_guess_ulp)
+
+
+def count_short_rcp_mismatch(first_bits: int, n: int, first_guess_ulp: int) -> int:
+    """See gpuk_oracle_count_short_rcp_mismatch."""
+    return lib().gpuk_oracle_count_short_rcp_mismatch(first_bits, n, first_guess_ulp)

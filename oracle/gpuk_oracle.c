@@ -349,3 +349,43 @@ int64_t gpuk_oracle_count_div_rcp_mismatch(const float *a, const float *b, int64
     }
     return bad;
 }
+
+/* Models of the short square-root and reciprocal sequences of the HIP kernels, checked here against the C library
+ * over every mantissa.  The device starts from v_sqrt_f32 / v_rcp_f32, which are documented to 1 ULP; the models
+ * start from the correctly rounded value moved by `first_guess_ulp` in {-1, 0, +1} ULPs, i.e. from every value the
+ * instruction may return, and must reach the correctly rounded result from each.
+ *
+ * Square root (the sequence LLVM emits for an fp32 sqrt on operands that need no rescaling): with s the first
+ * guess, take s-1ulp if v - (s-1ulp)*s <= 0, else s+1ulp if v - (s+1ulp)*s > 0, else s.
+ * Returns the number of v = bits first_bits .. first_bits + n - 1 whose result differs from sqrtf(v). */
+static inline float next_ulp(float f, int k) { return bits_f32(f32_bits(f) + (uint32_t)k); }
+
+int64_t gpuk_oracle_count_short_sqrt_mismatch(uint32_t first_bits, int64_t n, int first_guess_ulp) {
+    int64_t bad = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        const float v = bits_f32(first_bits + (uint32_t)i);
+        const float want = sqrtf(v);
+        float s = next_ulp(want, first_guess_ulp);
+        const float dn = next_ulp(s, -1), up = next_ulp(s, 1);
+        const float r_dn = fmaf(-dn, s, v), r_up = fmaf(-up, s, v);
+        if (r_dn <= 0.0f) s = dn;
+        else if (r_up > 0.0f) s = up;
+        if (f32_bits(s) != f32_bits(want)) ++bad;
+    }
+    return bad;
+}
+
+/* Reciprocal: y the first guess; one Newton step y += y*(1 - s*y); then the quotient correction of 1/s with that
+ * reciprocal: q = y, q += y*(1 - s*q).  Returns the number of s whose result differs from 1.0f / s. */
+int64_t gpuk_oracle_count_short_rcp_mismatch(uint32_t first_bits, int64_t n, int first_guess_ulp) {
+    int64_t bad = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        const float s = bits_f32(first_bits + (uint32_t)i);
+        const float want = 1.0f / s;
+        float y = next_ulp(want, first_guess_ulp);
+        y = fmaf(fmaf(-s, y, 1.0f), y, y);
+        const float q = fmaf(fmaf(-s, y, 1.0f), y, y);
+        if (f32_bits(q) != f32_bits(want)) ++bad;
+    }
+    return bad;
+}

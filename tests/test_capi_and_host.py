@@ -66,6 +66,12 @@ def test_argument_validation_needs_no_gpu():
     assert w(p, p, p, p, p, p, p, p, p, p, 1, 2, 2, 2, 2, 128, 0, 1e-6, 0, None, p, None) == 1  # missing output
     assert w(p, p, p, p, p, p, p, p, p, p, 0, 2, 2, 2, 2, 128, 0, 1e-6, 0, p, p, None) == 0    # empty batch
     assert L.gpuk_copy_bytes(p, p, 24, None) == 1 and L.gpuk_copy_bytes(p, p, 0, None) == 0
+    assert L.gpuk_read_bytes(p, 24, p, None) == 1 and L.gpuk_read_bytes(p, 0, p, None) == 0
+    assert L.gpuk_read_bytes(p, 32, None, None) == 1 and L.gpuk_read_bytes(p + 4, 32, p, None) == 3
+    assert L.gpuk_fill_bytes(p, 24, 1, None) == 1 and L.gpuk_fill_bytes(None, 32, 1, None) == 1
+    assert L.gpuk_fill_bytes(p, 0, 1, None) == 0 and L.gpuk_fill_bytes(p + 8, 32, 1, None) == 3
+    assert L.gpuk_empty_grid(4, 100, 0, None) == 1 and L.gpuk_empty_grid(4, 2048, 0, None) == 1
+    assert L.gpuk_empty_grid(4, 256, 1 << 20, None) == 1 and L.gpuk_empty_grid(0, 256, 0, None) == 0
     assert L.gpuk_set_tuning(b"no_such_knob", 1) == 1 and L.gpuk_set_tuning(b"norm_quant_nchunk", 3) == 1
     assert L.gpuk_set_tuning(b"norm_quant_nchunk", 0) == 0
 

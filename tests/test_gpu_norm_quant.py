@@ -393,6 +393,30 @@ def test_increment_floats_calibration_kernel(device):
         assert torch.equal(data.cpu(), want), n
 
 
+def test_one_direction_calibration_kernels(device):
+    """The write-only calibration kernel fills exactly the bytes asked for (guard bytes on both sides stay) with a
+    pattern that depends on the place; the read-only one and the empty grid write nothing."""
+    from gpuk_amd import capi
+
+    for nbytes in (16, 16 * 1024, 16 * 1024 + 48, 5 * 16 * 1024 - 16):
+        buf = torch.full((nbytes + 64,), 0x5A, dtype=torch.uint8, device=device)
+        capi.fill_bytes(buf[32:], nbytes, seed=7)
+        torch.cuda.synchronize()
+        host = buf.cpu()
+        assert (host[:32] == 0x5A).all() and (host[-32:] == 0x5A).all(), nbytes
+        words = host[32:-32].view(torch.int32).view(-1, 4)
+        place = torch.arange(words.shape[0], dtype=torch.int64)
+        base = (place // 1024) * 1024 + place % 256          # first 16-byte chunk of the lane that stored this one
+        assert torch.equal(words[:, 0].to(torch.int64) & 0xFFFFFFFF, (7 + base) & 0xFFFFFFFF), nbytes
+        assert (words[:, 3] == 7).all()
+        sink = torch.zeros(4, dtype=torch.int32, device=device)
+        before = buf.clone()
+        capi.read_bytes(buf[32:], nbytes, sink)
+        capi.empty_grid(37, 256, 6656)
+        torch.cuda.synchronize()
+        assert torch.equal(buf, before) and not sink.any()
+
+
 @pytest.mark.parametrize("fp8_max", [448.0, 240.0])
 def test_static_scale_too_small_saturates(device, fp8_max):
     """A static scale 8 times too small: most quotients exceed fp8_max and are clipped to it, as the oracle's clamp

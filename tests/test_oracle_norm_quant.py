@@ -184,3 +184,40 @@ def test_reciprocal_quotient_model_is_exact():
     for s in (2.0 ** -60, 0.0123, 1.0, 2.0 ** 60):
         bad += c_oracle.count_div_rcp_mismatch(special, torch.full_like(special, s))
     assert bad == 0
+
+
+def test_short_sqrt_and_reciprocal_models_are_exact():
+    """The kernels take sqrt and 1/x by v_sqrt_f32 / v_rcp_f32 (1 ULP) plus correction steps instead of the compiler's
+    general expansions.  The same sequences in C, started from every value within one ULP of the true result, give
+    the correctly rounded result for every mantissa (square root: both exponent parities), except the reciprocal of a
+    number whose mantissa bits are all ones, which the kernels send to the general division."""
+    import struct
+
+    bits = lambda f: struct.unpack("<I", struct.pack("<f", f))[0]
+    for first_guess in (-1, 0, 1):
+        for lo in (1.0, 2.0, 2.0 ** -41, 2.0 ** 58):
+            assert c_oracle.count_short_sqrt_mismatch(bits(lo), 1 << 23, first_guess) == 0, (lo, first_guess)
+        for lo in (1.0, 2.0 ** -30, 2.0 ** 29):
+            bad = c_oracle.count_short_rcp_mismatch(bits(lo), (1 << 23) - 1, first_guess)   # all but the all-ones mantissa
+            assert bad == 0, (lo, first_guess, bad)
+    assert c_oracle.count_short_rcp_mismatch(bits(1.0) + (1 << 23) - 1, 1, 1) == 1   # the excluded case does fail
+
+
+def test_quotients_by_row_length_and_by_fp8_max_are_exact():
+    """mean = sum / H and scale = amax / fp8_max are taken as one multiply and two fused multiply-adds with the
+    reciprocal rounded on the host: equal to the IEEE quotient for every row length that is a multiple of 8 up to
+    65536 (random sums on the guarded range) and for every positive bf16 amax on that range with 448 and 240."""
+    g = torch.Generator().manual_seed(21)
+    hs = torch.arange(8, 65536 + 8, 8, dtype=torch.float32)
+    bad = 0
+    for _ in range(40):
+        sums = torch.exp2(torch.rand(hs.numel(), generator=g) * 100 - 50).float()
+        bad += c_oracle.count_div_rcp_mismatch(sums.contiguous(), hs.contiguous())
+    for h in (7168.0, 5120.0, 12288.0, 1032.0, 65528.0):
+        sums = torch.exp2(torch.rand(1_000_000, generator=g) * 119 - 59.5).float()
+        bad += c_oracle.count_div_rcp_mismatch(sums, torch.full_like(sums, h))
+    allbf = torch.arange(1, 0x7F80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    amax = allbf[(allbf >= 2.0 ** -60) & (allbf < 2.0 ** 60)]
+    for fp8_max in (448.0, 240.0):
+        bad += c_oracle.count_div_rcp_mismatch(amax.contiguous(), torch.full_like(amax, fp8_max))
+    assert bad == 0
