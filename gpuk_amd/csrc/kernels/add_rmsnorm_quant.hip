@@ -77,7 +77,7 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
     using P = Pack16<T>;
     __shared__ float s_sum[kReduceSlots];
     __shared__ float s_max[kReduceSlots];
-    GPUK_STAMPS_BEGIN();  // profiling build only; slots: see kNormQuantStampNames
+    GPUK_STAMPS_BEGIN();  // profiling build only
 
     const int tid = threadIdx.x;
     const int num_waves = nthreads >> 6;

@@ -35,24 +35,14 @@ extern "C" int gpuk_set_tuning(const char *key, int value) {
         gpuk::set_norm_quant_tuning(5, value);
         return GPUK_OK;
     }
-    if (strcmp(key, "rope_walk") == 0) {
-        if (value < 0 || value > 2) return GPUK_ERR_INVALID_ARG;
-        gpuk::set_rope_tuning(1, value);
-        return GPUK_OK;
-    }
-    if (strcmp(key, "rope_walk_stream") == 0) {
+    if (strcmp(key, "rope_stream_rows") == 0) {
         if (value < 0 || value > 2) return GPUK_ERR_INVALID_ARG;
         gpuk::set_rope_tuning(3, value);
         return GPUK_OK;
     }
-    if (strcmp(key, "rope_walk_merge_rows") == 0) {
+    if (strcmp(key, "rope_merge_rows") == 0) {
         if (value < 0 || value > 1) return GPUK_ERR_INVALID_ARG;
         gpuk::set_rope_tuning(4, value);
-        return GPUK_OK;
-    }
-    if (strcmp(key, "rope_walk_waves") == 0) {
-        if (value < 0 || value > (1 << 20)) return GPUK_ERR_INVALID_ARG;
-        gpuk::set_rope_tuning(2, value);
         return GPUK_OK;
     }
     if (strcmp(key, "rope_block_threads") == 0) {

@@ -52,10 +52,9 @@ struct RopeArgs {
     float eps, k_scale, v_scale;
     // mRoPE: bit f of axis1 / axis2 set when rotary frequency f takes its position from axis 1 / 2
     uint32_t axis1[4], axis2[4];
-    // token-walking kernel: number of waves in the grid (token stride of a wave) and the token count
-    uint32_t walk_waves, num_tokens;
-    uint32_t walk_stream;  // 1: q_out / in-place stores (and in-place loads) bypass the L2; for large batches
-    uint32_t walk_merge_rows;  // mRoPE: every aligned group of 8 frequencies takes one axis: rows are merged on load
+    uint32_t num_tokens;
+    uint32_t stream_rows;  // 1: q_out / K rows / in-place rows are stored past the L2 (calls that move more than a few MB)
+    uint32_t merge_rows;   // mRoPE: every aligned group of 8 frequencies takes one axis: each lane loads from that axis's row
 };
 
 // dword mask selecting the 16-bit halves whose bit is set in a 2-bit field
@@ -277,7 +276,7 @@ struct RopeUnit {
         const int64_t p0 = st.p0;
         if constexpr (AXES == 3) {
             const int64_t p1 = st.p1, p2 = st.p2;
-            if (a.walk_merge_rows && (p1 != p0 || p2 != p0)) {
+            if (a.merge_rows && (p1 != p0 || p2 != p0)) {
                 // every aligned group of 8 frequencies takes one axis: each lane reads its pieces from that axis's row
                 const uint32_t b1 = trig_bits<D, NEOX>(a.axis1, sub), b2 = trig_bits<D, NEOX>(a.axis2, sub);
                 const int64_t pa = (b2 & 1u) ? p2 : ((b1 & 1u) ? p1 : p0);
@@ -334,7 +333,7 @@ struct RopeUnit {
         if (st.active && (st.is_q || slot_ok)) {
             if constexpr (!SETKV) {
                 uint16_t *dst = static_cast<uint16_t *>(a.qkv_out) + ((int64_t)st.t * heads_all + head) * D;
-                store_pair<HALF * 2>(dst + c0(sub), oa, ob, a.walk_stream != 0);
+                store_pair<HALF * 2>(dst + c0(sub), oa, ob, a.stream_rows != 0);
             } else if (KVFP8 && !st.is_q) {
                 uint8_t *dst = static_cast<uint8_t *>(a.k_cache) + (st.slot * a.hk + (head - a.hq)) * D;
                 const float s = a.k_scale, rcp = 1.0f / s;
@@ -349,7 +348,7 @@ struct RopeUnit {
                 // q_out row or (16-bit) K cache row of the slot: one store sequence, destination chosen per lane
                 uint16_t *dst = st.is_q ? static_cast<uint16_t *>(a.q_out) + ((int64_t)st.t * a.hq + head) * D
                                         : static_cast<uint16_t *>(a.k_cache) + (st.slot * a.hk + (head - a.hq)) * D;
-                store_pair<HALF * 2>(dst + c0(sub), oa, ob, a.walk_stream != 0);
+                store_pair<HALF * 2>(dst + c0(sub), oa, ob, a.stream_rows != 0);
             }
         }
 
@@ -400,7 +399,7 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
     a.hv = (int)(hv_and_waves & 0xffffffu);
     a.ps_token = ps_token;
     a.ps_axis = ps_axis;
-    GPUK_STAMPS_BEGIN();  // profiling build only; slots: see kRopeUnitStampNames
+    GPUK_STAMPS_BEGIN();  // profiling build only
     const int lane = threadIdx.x & 63;
     UnitState st;
     Unit::issue_loads(a, unit, lane, st);
@@ -415,528 +414,6 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
     GPUK_STAMP(4);          // rows stored (issued)
     GPUK_STAMP_DRAINED(5);  // ... and acknowledged
     GPUK_STAMPS_WRITE(unit);
-}
-
-// ---------------------------------------------------------------------------------------------------------------
-// Token-walking form for large batches.  A wave owns whole tokens (its first token is its wave index, the next one
-// walk_waves further on, ...) and walks each token's units in order.  What the one-wave-per-unit kernel above repeats
-// for every unit is done once per wave (norm weights unpacked to fp32) or once per token (position, slot, cos/sin row
-// loaded and unpacked), and the loads of the following kWalkRing units -- the first units of the wave's next token
-// included -- are in flight while the current one is finished, as is the next token's cos/sin row.  The grid is sized
-// to what the chip holds at once, so there is one dispatch round and no tail of partly filled rounds.
-//
-// Prefetched data travels global memory -> LDS directly (global_load_lds_dwordx4: lane l's 16 bytes land at
-// M0 + 16*l), so no register is the destination of a load in flight, and is waited for with an explicit
-// s_waitcnt vmcnt(N): left to the compiler, loop-carried load destinations get copied at every join (reading
-// registers whose data has not arrived) or the whole memory queue is drained at every step.  What makes the explicit
-// waits safe: N never exceeds the number of vector memory instructions issued after the transfer waited for (the
-// stores and loads the compiler emits only add to that number), vector memory instructions complete in issue order
-// on this target, and the LDS reads that follow a wait are ordinary loads the compiler orders after it (the wait
-// clobbers memory).  A staging buffer is refilled only after its previous content is in registers (in_registers()).
-constexpr int kWalkWaves = 4;  // waves per workgroup of the walking kernel
-constexpr int kWalkRing = 2;   // staging buffers per wave = units in flight beyond the current one
-
-// The base of a transfer has to sit in a pair of scalar registers.  It is wave-uniform by construction; reading it
-// through the first lane makes that hold for the compiler too, whatever it concluded about the loads the address was
-// computed from (for a value it already keeps in scalar registers the reads fold away).  "vcc" is named as clobbered
-// only to keep the allocator from handing it over as that operand, which the instruction does not take.
-__device__ __forceinline__ const void *in_scalar_registers(const void *p) {
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo);
-}
-// The transfers are self-sufficient about hardware hazards, because the compiler's hazard pass does not look inside
-// an asm statement: `s_nop 4` gives the five wait states a vector memory instruction needs after a v_readfirstlane
-// wrote the scalar registers it takes its base from (and the one it needs after M0 was written), and M0 is named as
-// clobbered, so that the compiler never carries a value of its own in M0 across a transfer (it answers with a
-// warning that M0 is a reserved register, silenced below: reserved means it allocates nothing there, which is the
-// point).
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-template <bool NT>
-__device__ __forceinline__ void lds_fill16(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
-    if constexpr (NT) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc", "m0");
-    } else {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc", "m0");
-    }
-}
-// the same for lanes 0-31 only: 512 bytes of LDS
-__device__ __forceinline__ void lds_fill16_lanes32(uint32_t lds_byte_offset, const void *wave_base, uint32_t lane_offset) {
-    uint64_t saved_exec;
-    asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_offset), "s"(in_scalar_registers(wave_base)) : "memory", "vcc", "m0");
-}
-// ... with a full address per lane (the lanes may read from different rows)
-__device__ __forceinline__ void lds_fill16_lanes32_gather(uint32_t lds_byte_offset, const void *lane_address) {
-    uint64_t saved_exec;
-    asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved_exec) : "s"(lds_byte_offset), "v"(lane_address) : "memory", "m0");
-}
-#pragma clang diagnostic pop
-template <int N>
-__device__ __forceinline__ void wait_fills() {  // until at most N vector memory instructions are outstanding
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-// wait_fills<n> for a run-time, wave-uniform n; larger values wait as for kMaxBehind (waiting for more is always safe)
-constexpr int kMaxBehind = 16;
-__device__ __forceinline__ void wait_fills_upto(uint32_t n) {
-    switch (n) {
-#define GPUK_WAIT_CASE(N) case N: wait_fills<N>(); break;
-        GPUK_WAIT_CASE(0) GPUK_WAIT_CASE(1) GPUK_WAIT_CASE(2) GPUK_WAIT_CASE(3) GPUK_WAIT_CASE(4) GPUK_WAIT_CASE(5)
-        GPUK_WAIT_CASE(6) GPUK_WAIT_CASE(7) GPUK_WAIT_CASE(8) GPUK_WAIT_CASE(9) GPUK_WAIT_CASE(10) GPUK_WAIT_CASE(11)
-        GPUK_WAIT_CASE(12) GPUK_WAIT_CASE(13) GPUK_WAIT_CASE(14) GPUK_WAIT_CASE(15)
-#undef GPUK_WAIT_CASE
-        default: wait_fills<kMaxBehind>(); break;
-    }
-}
-// Pins the point by which a value read from LDS is in registers: the transfers that refill the same LDS bytes are
-// issued after this statement (both are volatile), so they cannot overtake the read.
-__device__ __forceinline__ void in_registers(u32x4 &v) { asm volatile("" : "+v"(v)); }
-__device__ __forceinline__ uint32_t lds_offset_of(const void *shared_ptr) { return (uint32_t)(uintptr_t)shared_ptr; }
-
-// Same arithmetic as norm_rotate with the weights and the cos/sin values already unpacked to fp32.
-//   w[2j], w[2j+1]     : low / high half of dword j of the first chunk's weights;  w[8+2j], w[8+2j+1]: second chunk
-//   c[e], s[e]         : the lane's 8 cos / sin values in load_trig order
-template <typename T, int D, bool NEOX>
-__device__ __forceinline__ void norm_rotate_unpacked(const u32x4 &xa, const u32x4 &xb, const float (&w)[16],
-                                                     const float (&c)[8], const float (&s)[8], float eps, u32x4 &oa,
-                                                     u32x4 &ob) {
-    using P = Pack16<T>;
-    constexpr int LPH = D / 16;
-    float ss0 = 0.f, ss1 = 0.f;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        ss0 = P::add_squares(xa[j], ss0);
-        ss1 = P::add_squares(xb[j], ss1);
-    }
-    const float sumsq = group_allreduce<SumOp, LPH>(ss0 + ss1);
-    const float rstd = rsqrt_two_roundings(sumsq * (1.0f / D) + eps);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const float a0 = P::round(w[2 * j] * P::round(P::lo(xa[j]) * rstd));
-        const float a1 = P::round(w[2 * j + 1] * P::round(P::hi(xa[j]) * rstd));
-        const float b0 = P::round(w[8 + 2 * j] * P::round(P::lo(xb[j]) * rstd));
-        const float b1 = P::round(w[8 + 2 * j + 1] * P::round(P::hi(xb[j]) * rstd));
-        if constexpr (NEOX) {
-            const float cl = c[2 * j], ch = c[2 * j + 1], sl = s[2 * j], sh = s[2 * j + 1];
-            oa[j] = P::pack(P::round(a0 * cl) - P::round(b0 * sl), P::round(a1 * ch) - P::round(b1 * sh));
-            ob[j] = P::pack(P::round(b0 * cl) + P::round(a0 * sl), P::round(b1 * ch) + P::round(a1 * sh));
-        } else {
-            oa[j] = P::pack(P::round(a0 * c[j]) - P::round(a1 * s[j]), P::round(a1 * c[j]) + P::round(a0 * s[j]));
-            ob[j] = P::pack(P::round(b0 * c[4 + j]) - P::round(b1 * s[4 + j]),
-                            P::round(b1 * c[4 + j]) + P::round(b0 * s[4 + j]));
-        }
-    }
-}
-
-template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
-struct RopeWalk {
-    using P = Pack16<T>;
-    static constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
-    enum Kind { kQ = 0, kK = 1, kMixed = 2 };
-
-    const RopeArgs &a;
-    const int lane, sub, hl;
-    const int heads_qk, heads_all, v_chunks;
-    float wq[16], wk[16];  // norm weights of the lane's two chunks, fp32
-    float c[8], s[8];      // cos / sin of the current token
-    int64_t slot;          // cache slot of the current token
-    uint32_t t, u;         // current token and unit
-    int piece_axis;                         // mRoPE: axis of the 16-byte table-row piece this lane fetches
-
-    const void *const qkv_in, *const cos_sin;  // copies of the kernel's leading arguments, see rope_rms_walk_kernel
-
-    __device__ __forceinline__ RopeWalk(const RopeArgs &args, int lane_, const void *qkv_in_, const void *cos_sin_,
-                                        int heads_qk_, int heads_all_, int hv_)
-        : a(args), lane(lane_), sub(lane_ % LPH), hl(lane_ / LPH), heads_qk(heads_qk_), heads_all(heads_all_),
-          v_chunks(SETKV ? hv_ * (D / 8) : 0), qkv_in(qkv_in_), cos_sin(cos_sin_) {
-        if constexpr (AXES == 3) {
-            // first frequency of the lane's piece of a table row (cos pieces, then sin pieces); the bitmap words are
-            // picked with selects so that they stay in scalar registers (an index per lane would read them from memory)
-            const uint32_t f = 8 * (((uint32_t)lane % (D / 8)) % (D / 16));
-            auto bit = [&](const uint32_t (&bitmap)[4]) {
-                const uint32_t word = f < 32 ? bitmap[0] : (f < 64 ? bitmap[1] : (f < 96 ? bitmap[2] : bitmap[3]));
-                return (word >> (f & 31)) & 1u;
-            };
-            piece_axis = bit(a.axis2) ? 2 : (bit(a.axis1) ? 1 : 0);
-        }
-    }
-
-    __device__ __forceinline__ const uint16_t *token_row(uint32_t tt) const {
-        return static_cast<const uint16_t *>(qkv_in) + (int64_t)tt * heads_all * D;
-    }
-    __device__ __forceinline__ bool unit_has_v(uint32_t uu) const { return SETKV && (int)(uu * 64) < v_chunks; }
-
-    // Unit uu of token tt -> 2 KiB at LDS byte offset `stage`: the two 16-byte chunks of every lane (lanes past the
-    // last Q/K head re-read the last head).  Two transfers.
-    __device__ __forceinline__ void fill_unit(uint32_t stage, uint32_t tt, uint32_t uu) const {
-        const int head = min((int)(uu * HPW) + hl, heads_qk - 1);
-        const uint32_t off = (uint32_t)(head * D + 8 * sub) * 2u;
-        // streamed when the results go elsewhere; in place the same lines are written a moment later
-        // streamed when the results go elsewhere or the batch is large; in place and small, the same lines are
-        // written a moment later and are better kept
-        if (SETKV || a.walk_stream) {
-            lds_fill16<true>(stage, token_row(tt), off);
-            lds_fill16<true>(stage + 1024, token_row(tt), off + HALF * 2);
-        } else {
-            lds_fill16<false>(stage, token_row(tt), off);
-            lds_fill16<false>(stage + 1024, token_row(tt), off + HALF * 2);
-        }
-    }
-    // Unit uu's share of token tt's V row -> 1 KiB at `dst` (lanes past the row's end re-read its last chunk)
-    __device__ __forceinline__ void fill_v(uint32_t dst, uint32_t tt, uint32_t uu) const {
-        const int chunk = min((int)(uu * 64) + lane, v_chunks - 1);
-        lds_fill16<true>(dst, token_row(tt) + (int64_t)heads_qk * D, (uint32_t)chunk * 16u);
-    }
-    // Table row `pos` (2*D bytes: cos | sin) -> 512 bytes at `dst`, repeated 256/D times
-    __device__ __forceinline__ void fill_row(uint32_t dst, int64_t pos) const {
-        lds_fill16_lanes32(dst, static_cast<const uint16_t *>(cos_sin) + pos * D, (16u * lane) % (2u * D));
-    }
-    // mRoPE with every aligned group of 8 frequencies on one axis (chunked sections on multiples of 8): each lane
-    // fetches its 16-byte piece of the row from the table row of that group's axis, so the row arrives merged
-    __device__ __forceinline__ void fill_row_merged(uint32_t dst, int64_t p0, int64_t p1, int64_t p2) const {
-        const uint32_t piece = (uint32_t)lane % (D / 8);  // 16-byte piece of the row: cos pieces, then sin pieces
-        const int64_t pos = piece_axis == 2 ? p2 : (piece_axis == 1 ? p1 : p0);
-        lds_fill16_lanes32_gather(dst, static_cast<const char *>(cos_sin) + pos * (2 * D) + 16 * piece);
-    }
-    // Both weight vectors -> 1 KiB at `dst`: q weights in the first 512 bytes, k weights in the second
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-    __device__ __forceinline__ void fill_weights(uint32_t dst) const {
-        const char *qw = static_cast<const char *>(a.qw), *kw = static_cast<const char *>(a.kw);
-        // one transfer with per-lane addresses relative to qw: lanes 32-63 reach over to kw
-        const int64_t k_minus_q = kw - qw;
-        const uint32_t within = (16u * (lane & 31)) % (2u * D);
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(qw + (lane < 32 ? 0 : k_minus_q) + within) : "memory", "m0");
-    }
-#pragma clang diagnostic pop
-    __device__ __forceinline__ void take_weights(const unsigned char *at) {
-        u32x4 qa = *reinterpret_cast<const u32x4 *>(at + 16 * sub), qb = *reinterpret_cast<const u32x4 *>(at + D + 16 * sub);
-        u32x4 ka = *reinterpret_cast<const u32x4 *>(at + 512 + 16 * sub), kb = *reinterpret_cast<const u32x4 *>(at + 512 + D + 16 * sub);
-        in_registers(qa);
-        in_registers(qb);
-        in_registers(ka);
-        in_registers(kb);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            wq[2 * j] = P::lo(qa[j]);
-            wq[2 * j + 1] = P::hi(qa[j]);
-            wq[8 + 2 * j] = P::lo(qb[j]);
-            wq[8 + 2 * j + 1] = P::hi(qb[j]);
-            wk[2 * j] = P::lo(ka[j]);
-            wk[2 * j + 1] = P::hi(ka[j]);
-            wk[8 + 2 * j] = P::lo(kb[j]);
-            wk[8 + 2 * j + 1] = P::hi(kb[j]);
-        }
-    }
-
-    // the staged rows (512 bytes each) -> c[], s[] of the current token
-    __device__ __forceinline__ void take_table(const unsigned char *rows, bool split) {
-        auto row_cos = [&](int r) -> u32x4 {
-            const unsigned char *p = rows + 512 * r;
-            if constexpr (NEOX) {
-                return *reinterpret_cast<const u32x4 *>(p + 16 * sub);
-            } else {
-                const u32x2 lo = *reinterpret_cast<const u32x2 *>(p + 8 * sub);
-                const u32x2 hi = *reinterpret_cast<const u32x2 *>(p + D / 2 + 8 * sub);
-                return u32x4{lo[0], lo[1], hi[0], hi[1]};
-            }
-        };
-        auto row_sin = [&](int r) -> u32x4 {
-            const unsigned char *p = rows + 512 * r + D;
-            if constexpr (NEOX) {
-                return *reinterpret_cast<const u32x4 *>(p + 16 * sub);
-            } else {
-                const u32x2 lo = *reinterpret_cast<const u32x2 *>(p + 8 * sub);
-                const u32x2 hi = *reinterpret_cast<const u32x2 *>(p + D / 2 + 8 * sub);
-                return u32x4{lo[0], lo[1], hi[0], hi[1]};
-            }
-        };
-        u32x4 cv = row_cos(0), sv = row_sin(0);
-        in_registers(cv);
-        in_registers(sv);
-        if constexpr (AXES == 3) {
-            if (split) {
-                u32x4 c1 = row_cos(1), s1 = row_sin(1), c2 = row_cos(2), s2 = row_sin(2);
-                in_registers(c1);
-                in_registers(s1);
-                in_registers(c2);
-                in_registers(s2);
-                const uint32_t b1 = trig_bits<D, NEOX>(a.axis1, sub), b2 = trig_bits<D, NEOX>(a.axis2, sub);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t m1 = halves_mask(b1 >> (2 * j)), m2 = halves_mask(b2 >> (2 * j));
-                    cv[j] = bitselect(m2, c2[j], bitselect(m1, c1[j], cv[j]));
-                    sv[j] = bitselect(m2, s2[j], bitselect(m1, s1[j], sv[j]));
-                }
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            c[2 * j] = P::lo(cv[j]);
-            c[2 * j + 1] = P::hi(cv[j]);
-            s[2 * j] = P::lo(sv[j]);
-            s[2 * j + 1] = P::hi(sv[j]);
-        }
-    }
-
-    // Norm, rotation and stores of the current unit.  Returns nothing; the caller counts the store instructions:
-    // two per kind of lane present (Q, K with a valid slot), one for the V chunk.
-    template <int KIND>
-    __device__ __forceinline__ void finish_unit(const u32x4 &xa, const u32x4 &xb, const u32x4 &v, bool has_v, bool stream_q) {
-        const int head_raw = (int)(u * HPW) + hl;
-        const bool active = KIND == kQ || head_raw < heads_qk;
-        const bool is_q = KIND == kQ || (KIND == kMixed && head_raw < a.hq);
-        u32x4 oa, ob;
-        if constexpr (KIND == kQ) {
-            norm_rotate_unpacked<T, D, NEOX>(xa, xb, wq, c, s, a.eps, oa, ob);
-        } else if constexpr (KIND == kK) {
-            norm_rotate_unpacked<T, D, NEOX>(xa, xb, wk, c, s, a.eps, oa, ob);
-        } else {
-            float w[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) w[i] = is_q ? wq[i] : wk[i];
-            norm_rotate_unpacked<T, D, NEOX>(xa, xb, w, c, s, a.eps, oa, ob);
-        }
-        const bool slot_ok = !SETKV || slot >= 0;  // wave-uniform; a negative slot drops the token's K and V rows
-        if constexpr (!SETKV) {
-            if (active) {
-                uint16_t *dst = static_cast<uint16_t *>(a.qkv_out) + ((int64_t)t * heads_all + head_raw) * D + 8 * sub;
-                store_pair<HALF * 2>(dst, oa, ob, stream_q);
-            }
-        } else {
-            if (KIND != kK && is_q) {
-                uint16_t *dst = static_cast<uint16_t *>(a.q_out) + ((int64_t)t * a.hq + head_raw) * D + 8 * sub;
-                store_pair<HALF * 2>(dst, oa, ob, stream_q);
-            }
-            if (KIND != kQ && !is_q && active && slot_ok) {
-                const int64_t row = (slot * a.hk + (head_raw - a.hq)) * D + 8 * sub;
-                if constexpr (KVFP8) {
-                    uint8_t *dst = static_cast<uint8_t *>(a.k_cache) + row;
-                    const float sc = a.k_scale, rcp = 1.0f / sc;
-                    if (scale_is_fast(sc)) {
-                        *reinterpret_cast<u32x2 *>(dst) = quantize_chunk<T, true>(oa, sc, rcp);
-                        *reinterpret_cast<u32x2 *>(dst + HALF) = quantize_chunk<T, true>(ob, sc, rcp);
-                    } else {
-                        *reinterpret_cast<u32x2 *>(dst) = quantize_chunk<T, false>(oa, sc, rcp);
-                        *reinterpret_cast<u32x2 *>(dst + HALF) = quantize_chunk<T, false>(ob, sc, rcp);
-                    }
-                } else {
-                    uint16_t *dst = static_cast<uint16_t *>(a.k_cache) + row;
-                    *reinterpret_cast<u32x4 *>(dst) = oa;
-                    *reinterpret_cast<u32x4 *>(dst + HALF) = ob;
-                }
-            }
-            // V: chunk u*64 + lane of the token's row, copied or quantised (the host takes this kernel only when
-            // the units of a token cover the whole row: units_per_token * 64 >= chunks)
-            const int chunk = (int)(u * 64) + lane;
-            if (has_v && slot_ok && chunk < v_chunks) {
-                const int64_t off = slot * a.hv * D + 8 * (int64_t)chunk;
-                if constexpr (!KVFP8) {
-                    *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(a.v_cache) + off) = v;
-                } else {
-                    const float sc = a.v_scale, rcp = 1.0f / sc;
-                    *reinterpret_cast<u32x2 *>(static_cast<uint8_t *>(a.v_cache) + off) =
-                        scale_is_fast(sc) ? quantize_chunk<T, true>(v, sc, rcp) : quantize_chunk<T, false>(v, sc, rcp);
-                }
-            }
-        }
-    }
-};
-
-template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
-__global__ void __launch_bounds__(kWalkWaves * 64)
-rope_rms_walk_kernel(const int64_t *__restrict__ positions, const int64_t *__restrict__ kv_loc, const void *qkv_in,
-                     const void *cos_sin, uint32_t n_waves, uint32_t tokens, uint32_t upt, int heads_qk, int heads_all,
-                     int ps_token, int ps_axis, int hv, const RopeArgs a) {
-    // The arguments ahead of `a` are what a wave needs to issue its first transfers and the loads of its first
-    // positions.  (Having them preloaded into scalar registers at wave launch, -amdgpu-kernarg-preload-count, was
-    // measured: no difference.)
-    using Walk = RopeWalk<T, D, NEOX, AXES, SETKV, KVFP8>;
-    constexpr int HPW = Walk::HPW, RING = kWalkRing;
-    __shared__ u32x4 s_stage[kWalkWaves][RING][128];  // per wave: the staged units, 2 KiB each
-    __shared__ u32x4 s_v[kWalkWaves][64];             // per wave: one unit's V chunks
-    __shared__ u32x4 s_w[kWalkWaves][64];             // per wave: the norm weights, read once
-    __shared__ u32x4 s_rows[kWalkWaves][AXES * 32];   // per wave: the table rows of one token, 512 bytes each
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t first = blockIdx.x * kWalkWaves + wave;
-    if (first >= n_waves) return;  // the host keeps the number of waves <= the number of tokens
-    GPUK_STAMPS_BEGIN();  // profiling build only; slots: see kRopeWalkStampNames
-    Walk w(a, threadIdx.x & 63, qkv_in, cos_sin, heads_qk, heads_all, hv);
-    w.t = first;
-    w.u = 0;
-    const uint32_t stage_at = lds_offset_of(&s_stage[wave][0][0]), v_at = lds_offset_of(&s_v[wave][0]),
-                   rows_at = lds_offset_of(&s_rows[wave][0]), weights_at = lds_offset_of(&s_w[wave][0]);
-
-    auto load_positions = [&](uint32_t tt, int64_t &p0, int64_t &p1, int64_t &p2) {
-        p0 = positions[(int64_t)tt * ps_token];
-        if constexpr (AXES == 3) {
-            p1 = positions[ps_axis + (int64_t)tt * ps_token];
-            p2 = positions[2 * (int64_t)ps_axis + (int64_t)tt * ps_token];
-        } else {
-            p1 = p2 = p0;
-        }
-    };
-    // `issued` counts the vector memory instructions this wave is known to have issued (transfers, and the stores
-    // of finished units); a mark is its value right after the transfers of one staged unit / V share / table row set.
-    // Waiting until at most issued - mark instructions are outstanding waits for exactly those transfers.
-    uint32_t issued = 0, rows_mark = 0, v_mark = 0;
-    uint32_t mark[RING];  // mark[0]: the current unit, mark[i]: the unit i further on
-    bool split = false;   // the three position axes of the token whose rows are staged differ
-    auto fill_table = [&](int64_t p0, int64_t p1, int64_t p2) {
-        if constexpr (AXES == 3) {
-            if (a.walk_merge_rows && (p1 != p0 || p2 != p0)) {  // one transfer brings the merged row
-                split = false;
-                w.fill_row_merged(rows_at, p0, p1, p2);
-                issued += 1;
-                rows_mark = issued;
-                return;
-            }
-        }
-        w.fill_row(rows_at, p0);
-        issued += 1;
-        if constexpr (AXES == 3) {
-            split = p1 != p0 || p2 != p0;  // wave-uniform; text tokens carry three equal positions
-            if (split) {
-                w.fill_row(rows_at + 512, p1);
-                w.fill_row(rows_at + 1024, p2);
-                issued += 2;
-            }
-        }
-        rows_mark = issued;
-    };
-    // (ft, fu): the next unit to stage; fslot: the staging buffer it goes to
-    uint32_t ft = first, fu = 0, fslot = 0;
-    bool fmore = true;
-    auto stage_next = [&]() {
-        if (fmore) {
-            w.fill_unit(stage_at + fslot * 2048, ft, fu);
-            issued += 2;
-            if (++fu == upt) {
-                fu = 0;
-                ft += n_waves;
-                fmore = ft < tokens;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i + 1 < RING; ++i) mark[i] = mark[i + 1];
-        mark[RING - 1] = issued;
-        fslot = fslot + 1 == (uint32_t)RING ? 0 : fslot + 1;
-    };
-
-    // prologue.  The loads of the first positions are issued first and waited for only after the transfers that do
-    // not need them (weights, the first unit, its V share) are on their way; the first token's table row follows,
-    // ahead of the remaining staged units: memory operations complete in issue order, so the first unit can start as
-    // soon as its own data and the row are there, not after everything staged behind them.
-    {   // every kernel argument the transfers below take is in registers before the position loads are issued: a
-        // wait for an argument fetched later would also wait for the positions (scalar loads return in any order,
-        // so the only wait there is waits for all of them)
-        const void *qw_ = a.qw, *kw_ = a.kw;
-        asm volatile("" ::"s"(qkv_in), "s"(cos_sin), "s"(qw_), "s"(kw_), "s"(tokens), "s"(upt), "s"(heads_qk), "s"(heads_all), "s"(hv));
-    }
-    int64_t p0, p1, p2, np0 = 0, np1 = 0, np2 = 0;
-    load_positions(first, p0, p1, p2);
-    int64_t slot_next = SETKV ? kv_loc[first] : 0;
-    if (first + n_waves < tokens) load_positions(first + n_waves, np0, np1, np2);
-    w.fill_weights(weights_at);
-    issued += 1;
-    const uint32_t weights_mark = issued;
-#pragma unroll
-    for (int i = 0; i < RING; ++i) mark[i] = 0;
-    stage_next();
-    if (w.unit_has_v(0)) {
-        w.fill_v(v_at, first, 0);
-        issued += 1;
-        v_mark = issued;
-    }
-    fill_table(p0, p1, p2);
-#pragma unroll
-    for (int i = 1; i < RING; ++i) stage_next();
-    GPUK_STAMP(1);  // every transfer of the prologue issued (the first position has arrived)
-    wait_fills_upto(__builtin_amdgcn_readfirstlane(issued - weights_mark));
-    w.take_weights(reinterpret_cast<const unsigned char *>(&s_w[wave][0]));
-    GPUK_STAMP(2);  // norm weights arrived and unpacked
-    [[maybe_unused]] uint32_t units_done = 0;
-
-    // One step: wait for the current unit's transfers (and, at a token's first unit, for its table rows), move it to
-    // registers, refill what that freed (next token's rows, next unit's V share, the unit RING ahead), finish the unit.
-    uint32_t cslot = 0;  // staging buffer of the current unit
-    const bool stream_q = a.walk_stream != 0;
-    for (;;) {
-        const bool cur_v = w.unit_has_v(w.u), token_start = w.u == 0;
-        uint32_t newest = mark[0];  // the newest transfer this step reads
-        if (cur_v) newest = max(newest, v_mark);
-        if (token_start) newest = max(newest, rows_mark);
-        wait_fills_upto(__builtin_amdgcn_readfirstlane(issued - newest));  // uniform anyway; keeps the switch scalar
-#ifdef GPUK_STAMPS
-        if (units_done == 0) GPUK_STAMP(3);  // the first unit and its table row arrived
-#endif
-        const u32x4 *stage = &s_stage[wave][0][0] + cslot * 128;
-        u32x4 xa = stage[w.lane], xb = stage[64 + w.lane], v = u32x4{0, 0, 0, 0};
-        in_registers(xa);
-        in_registers(xb);
-        if (cur_v) {
-            v = s_v[wave][w.lane];
-            in_registers(v);
-        }
-        if (token_start) {
-            w.slot = slot_next;
-            w.take_table(reinterpret_cast<const unsigned char *>(&s_rows[wave][0]), split);
-            const uint32_t tn = w.t + n_waves;
-            if (tn < tokens) {
-                fill_table(np0, np1, np2);
-                if constexpr (SETKV) slot_next = kv_loc[tn];
-                if (tn + n_waves < tokens) load_positions(tn + n_waves, np0, np1, np2);
-            }
-        }
-        {   // the following unit's V share, before the unit RING ahead: a wait for it must not cover that one
-            uint32_t nu = w.u + 1, nt = w.t;
-            if (nu == upt) {
-                nu = 0;
-                nt += n_waves;
-            }
-            if (nt < tokens && w.unit_has_v(nu)) {
-                w.fill_v(v_at, nt, nu);
-                issued += 1;
-                v_mark = issued;
-            }
-        }
-        stage_next();  // refills the buffer just read; mark[0] now belongs to the following unit
-
-        const uint32_t h0 = w.u * HPW;
-        const bool slot_ok = !SETKV || w.slot >= 0;
-        if (h0 + HPW <= (uint32_t)a.hq) {
-            w.template finish_unit<Walk::kQ>(xa, xb, v, cur_v, stream_q);
-            issued += 2;
-        } else if (h0 >= (uint32_t)a.hq) {
-            w.template finish_unit<Walk::kK>(xa, xb, v, cur_v, stream_q);
-            issued += slot_ok ? 2 : 0;
-        } else {
-            // Lanes of both kinds, or Q lanes beside lanes past the last head.  Only stores that some lane takes part
-            // in are counted: with no lane active a store sequence may be branched over, and a count above what was
-            // issued would let a later wait return before its transfer has landed.
-            w.template finish_unit<Walk::kMixed>(xa, xb, v, cur_v, stream_q);
-            const bool has_k_lane = (uint32_t)a.hq < min(h0 + (uint32_t)HPW, (uint32_t)heads_qk);
-            issued += SETKV && slot_ok && has_k_lane ? 4 : 2;  // in place one store sequence serves both kinds of lanes
-        }
-        if (SETKV && cur_v && slot_ok) issued += 1;
-#ifdef GPUK_STAMPS
-        // the stores of the wave's first eight units issued: slots 4 .. 11 (a select chain: the slot is not a constant)
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-            if (units_done == (uint32_t)k) GPUK_STAMP(4 + k);
-        ++units_done;
-#endif
-        cslot = cslot + 1 == (uint32_t)RING ? 0 : cslot + 1;
-        if (++w.u == upt) {
-            w.u = 0;
-            w.t += n_waves;
-            if (w.t >= tokens) break;
-        }
-    }
-    GPUK_STAMP_DRAINED(12);  // every store of the wave acknowledged
-    GPUK_STAMPS_WRITE(first);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1245,103 +722,46 @@ int launch_2way_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned ba
     }
 }
 
-int g_block_threads = 0;    // 0 = default
-int g_walk = 0;             // token-walking kernel: 0 = built-in rule, 1 = never, 2 = always
-int g_walk_waves = 0;       // waves the walking grid may hold at once (0 = built-in)
-int g_walk_stream = 0;      // streaming stores of the walking kernel: 0 = built-in rule, 1 = never, 2 = always
-int g_walk_merge_rows = 0;  // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
+int g_block_threads = 0;  // 0 = default
+int g_stream_rows = 0;    // output rows stored past the L2: 0 = built-in rule, 1 = never, 2 = always
+int g_merge_rows = 0;     // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
 
+// Streaming stores, measured on MI355X (32/8/8, 28/4/4 and 64/8/8 heads, head sizes 64-256, random slots): q_out /
+// K rows / in-place rows written past the L2 are ahead from about 10 MB per call on (64+8 heads, fp8 cache: 5.9
+// against 7.0 us at 512 tokens, 16.0 against 18.1 at 2048; 40 heads: 19.0 against 21.1 us at 4096 tokens, 65.2 against
+// 80.2 at 16384; level at 5 MB and below) -- what a kernel leaves dirty in the L2 is written back at its end.
+constexpr int64_t kStreamFromBytes = 8'000'000;
 
-// Which kernel and which stores, measured on MI355X (32/8/8, 28/4/4 and 64/8/8 heads, head sizes 64-256, random slots):
-//   streaming stores : in the one-wave-per-unit kernel, q_out / K rows / in-place rows written past the L2 are ahead
-//                      from about 10 MB per call on (64+8 heads, fp8 cache: 5.9 against 7.0 us at 512 tokens, 16.0
-//                      against 18.1 at 2048; 40 heads: 19.0 against 21.1 us at 4096 tokens, 65.2 against 80.2 at
-//                      16384; level at 5 MB and below) -- what a kernel leaves dirty in the L2 is written back at its
-//                      end.  The walking kernel keeps its rows in the L2 up to 130 MB per call (18.5 against 19.1 us
-//                      at 4096 x 40 heads) and streams them (in place: loads too) above (27.5 against 27.9 us at
-//                      8192 x 32 heads, 35.1 against 41.2 at 8192 x 40);
-//   token-walking    : every wave walks ceil(T / capacity) tokens, and the grid's waves are dealt evenly to the
-//                      chip's 1024 SIMDs, so its run time moves in steps of ceil(waves / 1024) waves per SIMD (one
-//                      token per wave, 40 heads: 9.2 us at 1024 tokens, 12.1 at 2048, 15.4 at 3072, 19.0 at 4096,
-//                      and 14.5-14.8 anywhere from 2400 to 2800) while the other kernel's grows with the tokens.
-//                      Against the other kernel with streaming stores it is ahead only when writing a 16-bit cache,
-//                      with one position axis, head size 128 and one token per wave on a grid whose last step is full
-//                      with three or four waves on every SIMD (40 heads: 18.45 against 18.9 us at 4096 tokens, 14.9
-//                      against 15.1 at 3072).  In place the other kernel, its loads streamed as well, is ahead at
-//                      every size (40 heads: 12.4 against 14.2 us at 3000 tokens, 15.8 against 20.0 at 4096, 28.4
-//                      against 32.7 at 8192).  Elsewhere it is level or ahead too: 33.6
-//                      against 35.8 us at 8192 x 40 heads, 64.8 against 69.0 at 16384, 28.0 against 31.5 at 4096 x 72
-//                      heads with an fp8 cache, 65.6 against 70.7 at 8192 x 40 heads of 256, with three position axes
-//                      27.0 against 27.7 at 8192 x 32 heads and 50.7 against 51.9 at 16384 (16.5 both at 4096 with
-//                      an fp8 cache), and by 10-20 % where the walking grid's last step is thin (19.1 against 22.9 us
-//                      at 4100 tokens);
-//   one wave per unit: everything else.
-// (Cutting a token's units into runs shared by neighbouring waves, to fill the slots at any T, was measured too: it
-// narrows the walking kernel's dips -- 22.1 us at 4608 -- but never beats the better of the two kernels.)
-constexpr int64_t kWalkMinUnits = 10000;
-constexpr int64_t kWalkStreamBytes = 130'000'000;
-constexpr int64_t kUnitStreamBytes = 8'000'000;
-constexpr uint32_t kWalkCapacity = 4096;  // waves the chip holds at once at 4 per SIMD: one dispatch round
-constexpr uint32_t kComputeUnits = 256;   // MI355X
-
-// What a call of the 16-bit rope kernels launches: which kernel, its grid, whether the output rows go past the L2.
+// What a call of the 16-bit rope kernel launches: its grid, and whether the output rows go past the L2.
 struct RopePlan {
-    bool walk;                  // token-walking kernel (else one wave per unit)
-    uint32_t walk_waves;        // its grid, in waves
-    uint32_t threads, blocks;   // workgroup size and count of the launch
-    bool stream;                // q_out / K rows / in-place rows stored past the L2
+    uint32_t threads, blocks;  // workgroup size and count of the launch
+    bool stream;               // q_out / K rows / in-place rows stored past the L2
 };
 
-RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8) {
+RopePlan plan_rope(const RopeArgs &a, int D, bool set_kv, bool kv_fp8) {
     RopePlan p{};
-    // the walking kernel shares a token's V row out over the token's units, one 16-byte chunk per lane and unit
-    const bool v_fits = !set_kv || (int64_t)a.units_per_token * 64 >= (int64_t)a.hv * (D / 8);
-    const bool strides_fit = a.ps_token == (int)a.ps_token && a.ps_axis == (int)a.ps_axis;  // passed as 32-bit
-    // every wave the same number of tokens (the last ones one fewer)
-    const uint32_t capacity = g_walk_waves ? (uint32_t)g_walk_waves : kWalkCapacity;
-    const uint32_t tokens_per_wave = (a.num_tokens + capacity - 1) / capacity;
-    p.walk_waves = (a.num_tokens + tokens_per_wave - 1) / tokens_per_wave;
-    const uint32_t simds = 4 * kComputeUnits;
-    const uint32_t waves_per_simd = (p.walk_waves + simds - 1) / simds;  // of the fullest SIMD
-    const bool last_step_full = waves_per_simd >= 3 && 100 * (uint64_t)p.walk_waves >= 95 * (uint64_t)waves_per_simd * simds;
-    const bool slots_filled = last_step_full && set_kv && axes == 1 && !kv_fp8 && D == 128 && tokens_per_wave == 1;
-    p.walk = v_fits && strides_fit &&
-             (g_walk == 2 || (g_walk == 0 && (int64_t)a.total_units >= kWalkMinUnits && slots_filled));
     // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
     const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
     const int64_t call_bytes = set_kv ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
                                             (kv_fp8 ? 1 : 2) * ((int64_t)a.num_tokens * a.hk * D + elems_v)
                                       : 4 * elems_qk;
-    const int64_t stream_from = p.walk ? kWalkStreamBytes : kUnitStreamBytes;
-    p.stream = g_walk_stream == 2 || (g_walk_stream == 0 && call_bytes >= stream_from);
-    if (p.walk) {
-        p.threads = kWalkWaves * 64;
-        p.blocks = (p.walk_waves + kWalkWaves - 1) / kWalkWaves;
-    } else {
-        // Workgroup size, swept over 64/128/256/512 lanes and one workgroup per token for 2-9 units per token: four
-        // waves where a workgroup then holds whole tokens (its waves share the token's position and table row in the
-        // CU's caches: 3-15 % ahead at 28+4 heads) and for large batches (1-3 % ahead from 4096 tokens on), single
-        // waves for small batches of other head counts (2-6 % ahead at 64+8 heads with an fp8 cache up to 512 tokens,
-        // within 1-3 % either way for 3, 5 and 6 units per token); 128 lanes is the slowest in most cases.
-        p.threads = g_block_threads ? (uint32_t)g_block_threads : (a.units_per_token % 4 == 0 || a.total_units > 8192 ? 256u : 64u);
-        const uint32_t units_per_block = p.threads / 64;
-        p.blocks = (a.total_units + units_per_block - 1) / units_per_block;
-    }
+    p.stream = g_stream_rows == 2 || (g_stream_rows == 0 && call_bytes >= kStreamFromBytes);
+    // Workgroup size, swept over 64/128/256/512 lanes and one workgroup per token for 2-9 units per token: four
+    // waves where a workgroup then holds whole tokens (its waves share the token's position and table row in the
+    // CU's caches: 3-15 % ahead at 28+4 heads) and for large batches (1-3 % ahead from 4096 tokens on), single
+    // waves for small batches of other head counts (2-6 % ahead at 64+8 heads with an fp8 cache up to 512 tokens,
+    // within 1-3 % either way for 3, 5 and 6 units per token); 128 lanes is the slowest in most cases.
+    p.threads = g_block_threads ? (uint32_t)g_block_threads : (a.units_per_token % 4 == 0 || a.total_units > 8192 ? 256u : 64u);
+    const uint32_t units_per_block = p.threads / 64;
+    p.blocks = (a.total_units + units_per_block - 1) / units_per_block;
     return p;
 }
 
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 int launch_one(const RopeArgs &a, hipStream_t stream) {
-    const RopePlan p = plan_rope(a, D, AXES, SETKV, KVFP8);
+    const RopePlan p = plan_rope(a, D, SETKV, KVFP8);
     RopeArgs b = a;
-    b.walk_stream = p.stream ? 1u : 0u;
-    if (p.walk) {
-        b.walk_waves = p.walk_waves;
-        rope_rms_walk_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<p.blocks, p.threads, 0, stream>>>(
-            a.positions, a.kv_loc, a.qkv_in, a.cos_sin, b.walk_waves, a.num_tokens, a.units_per_token, a.hq + a.hk,
-            a.hq + a.hk + a.hv, (int)a.ps_token, (int)a.ps_axis, a.hv, b);
-        return hip_status(hipGetLastError());
-    }
+    b.stream_rows = p.stream ? 1u : 0u;
     const uint32_t log2_waves = p.threads == 64 ? 0u : p.threads == 128 ? 1u : p.threads == 256 ? 2u : 3u;
     rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<p.blocks, p.threads, 0, stream>>>(
         a.qkv_in, a.positions, a.total_units, a.units_per_token, a.upt_magic, a.hq, a.hk,
@@ -1447,12 +867,12 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
         if (section[0] < 0 || section[1] < 0 || section[2] < 0 || section[0] + section[1] + section[2] != D / 2)
             return GPUK_ERR_INVALID_ARG;
         build_axis_bitmaps(section, interleaved != 0, (int)(D / 2), a.axis1, a.axis2);
-        a.walk_merge_rows = 1;
+        a.merge_rows = 1;
         for (int f = 0; f < D / 2; f += 8) {
             const uint32_t g1 = (a.axis1[f >> 5] >> (f & 31)) & 0xffu, g2 = (a.axis2[f >> 5] >> (f & 31)) & 0xffu;
-            if ((g1 != 0 && g1 != 0xffu) || (g2 != 0 && g2 != 0xffu)) a.walk_merge_rows = 0;
+            if ((g1 != 0 && g1 != 0xffu) || (g2 != 0 && g2 != 0xffu)) a.merge_rows = 0;
         }
-        if (g_walk_merge_rows == 1) a.walk_merge_rows = 0;
+        if (g_merge_rows == 1) a.merge_rows = 0;
     }
     if (T == 0 || hq + hk + (set_kv ? hv : 0) == 0) return GPUK_OK;
     if (!qkv_in || !qw || !kw || !cos_sin || !positions) return GPUK_ERR_INVALID_ARG;
@@ -1464,7 +884,7 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
         if (!aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache)) return GPUK_ERR_MISALIGNED;
         if (kv_fp8 && !(k_scale > 0.f && v_scale > 0.f)) return GPUK_ERR_INVALID_ARG;
     }
-    // one wave (or one step of a walking wave) per group of 64/(D/16) consecutive Q/K heads of a token
+    // one wave per group of 64/(D/16) consecutive Q/K heads of a token
     const int64_t hpw = 64 / (D / 16);
     int64_t upt = (hq + hk + hpw - 1) / hpw;
     if (hq + hk == 0) return GPUK_ERR_UNSUPPORTED;  // a qkv row without Q and K heads has nothing to rotate
@@ -1502,10 +922,10 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
 }
 
 int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, int n_axes, int dtype, bool set_kv,
-                      int kv_dtype, int *walking, int *workgroups, int *lanes, int *streamed) {
+                      int kv_dtype, int *workgroups, int *lanes, int *streamed) {
     if (T <= 0 || hq < 0 || hk < 0 || hv < 0 || hq + hk == 0 || (n_axes != 1 && n_axes != 3)) return GPUK_ERR_INVALID_ARG;
     if (D != 64 && D != 128 && D != 256) return GPUK_ERR_UNSUPPORTED;
-    if (!walking || !workgroups || !lanes || !streamed) return GPUK_ERR_INVALID_ARG;
+    if (!workgroups || !lanes || !streamed) return GPUK_ERR_INVALID_ARG;
     if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32 && dtype != GPUK_DTYPE_F64) return GPUK_ERR_UNSUPPORTED;
     const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
     const int64_t hpw = 64 / (D / 16);
@@ -1518,16 +938,13 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
     a.hq = (int)hq;
     a.hk = (int)hk;
     a.hv = (int)hv;
-    a.ps_token = 1;  // positions as the wrappers pass them: strides that fit 32 bits
     if (wide) {
-        *walking = 0;
         *workgroups = (int)((a.total_units + 3) / 4);
         *lanes = 256;
         *streamed = 1;  // the fp32 / fp64 kernel always stores its rotated rows past the L2
         return GPUK_OK;
     }
-    const RopePlan p = plan_rope(a, (int)D, n_axes, set_kv, set_kv && kv_dtype == GPUK_KV_E4M3FN);
-    *walking = p.walk ? 1 : 0;
+    const RopePlan p = plan_rope(a, (int)D, set_kv, set_kv && kv_dtype == GPUK_KV_E4M3FN);
     *workgroups = (int)p.blocks;
     *lanes = (int)p.threads;
     *streamed = p.stream ? 1 : 0;
@@ -1538,10 +955,8 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
 
 void set_rope_tuning(int key, int value) {
     if (key == 0) g_block_threads = value;
-    if (key == 1) g_walk = value;
-    if (key == 2) g_walk_waves = value;
-    if (key == 3) g_walk_stream = value;
-    if (key == 4) g_walk_merge_rows = value;
+    if (key == 3) g_stream_rows = value;
+    if (key == 4) g_merge_rows = value;
 }
 
 }  // namespace gpuk
@@ -1551,10 +966,10 @@ GPUK_STAMPS_SETTER(gpuk_stamps_set_rope)
 
 extern "C" int gpuk_rope_rms_launch_shape(int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k,
                                           int64_t num_heads_v, int64_t head_size, int n_axes, int dtype, int set_kv,
-                                          int kv_dtype, int *walking, int *workgroups, int *lanes_per_workgroup,
+                                          int kv_dtype, int *workgroups, int *lanes_per_workgroup,
                                           int *streamed) {
     return gpuk::rope_launch_shape(num_tokens, num_heads_q, num_heads_k, num_heads_v, head_size, n_axes, dtype,
-                                   set_kv != 0, kv_dtype, walking, workgroups, lanes_per_workgroup, streamed);
+                                   set_kv != 0, kv_dtype, workgroups, lanes_per_workgroup, streamed);
 }
 
 extern "C" int gpuk_rope_rms(void *qkv, const void *qw, const void *kw, const void *cos_sin, const int64_t *positions,
@@ -1630,7 +1045,7 @@ extern "C" int gpuk_rope_rms_2way(const void *q0, const void *k0, const void *q1
     a.eps = eps;
     {   // as in the one-wave-per-unit rope kernel: streamed stores are ahead from about 10 MB per call on
         const int64_t call_bytes = 4 * batch_size * (num_tokens0 + num_tokens1) * (num_heads_q + num_heads_k) * head_size;
-        a.stream = g_walk_stream == 2 || (g_walk_stream == 0 && call_bytes >= kUnitStreamBytes) ? 1u : 0u;
+        a.stream = g_stream_rows == 2 || (g_stream_rows == 0 && call_bytes >= kStreamFromBytes) ? 1u : 0u;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool neox = !is_interleaved;  // reference: fused_rope.cpp:168-227 dispatches the NeoX kernel when !is_interleaved

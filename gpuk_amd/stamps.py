@@ -3,7 +3,7 @@
 100 MHz wall clock at its entry and exit, and its place on the chip.
 
     python -m gpuk_amd.stamps norm_quant [--tokens 1 128 512] [--hidden 7168]
-    python -m gpuk_amd.stamps rope [--config c3|c4|c5] [--tokens N] [--walk 0|1|2]
+    python -m gpuk_amd.stamps rope [--config c3|c4|c5] [--tokens N]
 
 Prints, per phase, how long the waves of one launch spent in it (ns: median, 10th and 90th percentile over waves;
 cycles are turned into ns with each launch's own ratio of wall-clock ticks to cycles), when waves start, first store
@@ -44,21 +44,12 @@ NORM_QUANT_PHASES = [
     (9, 10, "-> every store acknowledged"),
 ]
 ROPE_UNIT_PHASES = [
-    (0, 1, "entry -> activations, weights, position and slot requested"),
-    (1, 2, "-> position arrived, cos/sin requested"),
+    (0, 1, "entry -> activations and position requested, position and argument block arrived, weights and slot requested"),
+    (1, 2, "-> cos/sin requested"),
     (2, 3, "-> everything landed"),
     (3, 4, "-> norm, rotation, rows stored (issued)"),
     (4, 5, "-> every store acknowledged"),
 ]
-ROPE_WALK_PHASES = [
-    (0, 1, "entry -> prologue transfers issued (the first position has arrived)"),
-    (1, 2, "-> norm weights arrived and unpacked"),
-    (2, 3, "-> first unit and its table row arrived"),
-    (3, 4, "-> first unit finished, stores issued"),
-] + [(3 + k, 4 + k, f"-> unit {k + 1} finished, stores issued") for k in range(1, 8)] + [
-    (-1, 12, "last recorded unit -> every store acknowledged"),
-]
-
 
 def bind():
     if not os.path.exists(STAMPS_LIB):
@@ -98,13 +89,8 @@ def summarize(buf: torch.Tensor, phases, title: str):
           f"p90 {q(ticks, .9) * .01:6.2f}")
     total = 0.0
     for a, b, name in phases:
-        if a == -1:   # from the last unit stamp recorded
-            prev = torch.where(t[:, 4:12] != 0, t[:, 4:12], torch.zeros_like(t[:, 4:12])).max(dim=1).values
-            ok = (prev != 0) & (t[:, b] != 0)
-            dur = (t[ok, b] - prev[ok]).double() * ns_per_cycle
-        else:
-            ok = (t[:, a] != 0) & (t[:, b] != 0)
-            dur = (t[ok, b] - t[ok, a]).double() * ns_per_cycle
+        ok = (t[:, a] != 0) & (t[:, b] != 0)
+        dur = (t[ok, b] - t[ok, a]).double() * ns_per_cycle
         if dur.numel() == 0:
             continue
         total += q(dur, .5)
@@ -144,7 +130,7 @@ def run_norm_quant(L, tokens_list, hidden, quant):
         assert L.gpuk_stamps_set_norm_quant(None, 0) == 0
 
 
-def run_rope(L, config, tokens, walk):
+def run_rope(L, config, tokens):
     dev = torch.device("cuda:0")
     if config == "c3":
         r = workloads.config3(num_tokens=tokens) if tokens else workloads.config3()
@@ -153,9 +139,8 @@ def run_rope(L, config, tokens, walk):
     else:
         r = workloads.config5_rope(tokens or 128)
     T = r.num_tokens
-    capi.set_tuning("rope_walk", walk)
     n_axes = 3 if r.mrope_section is not None else 1
-    walking, groups, lanes, streamed = capi.rope_rms_launch_shape(T, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
+    groups, lanes, streamed = capi.rope_rms_launch_shape(T, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
                                                                   n_axes, torch.bfloat16, True, r.kv_dtype == torch.float8_e4m3fn)
     waves = groups * (lanes // 64)
     buf = torch.zeros((waves, SLOTS), dtype=torch.int64, device=dev)
@@ -173,25 +158,10 @@ def run_rope(L, config, tokens, walk):
         capi.rope_rms_set_kv(qkv, qw, kw, cs, pos, T, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size, r.is_neox,
                              r.eps, q_out, kc, vc, loc, r.k_scale, r.v_scale, r.mrope_section, r.is_interleaved)
     torch.cuda.synchronize()
-    title = (f"{'rope_rms_walk_kernel' if walking else 'rope_rms_kernel'}, {config} T={T} heads "
-             f"{r.num_heads_q}/{r.num_heads_k}/{r.num_heads_v}, {groups} workgroups x {lanes} lanes, "
-             f"rows stored {'past' if streamed else 'through'} the L2")
-    host = buf.cpu()
-    summarize(host, ROPE_WALK_PHASES if walking else ROPE_UNIT_PHASES, title)
-    if walking:
-        d = host[host[:, SLOTS - 3] != 0]
-        base = d[:, SLOTS - 3].min()
-        # when the stores of each unit left, on the launch's clock: entry (wall) + cycles since entry
-        ticks = (d[:, SLOTS - 2] - d[:, SLOTS - 3]).double()
-        cyc = (d[:, 12] - d[:, 0]).double()
-        ratio = float((ticks * 10).sum() / cyc.sum())
-        start = (d[:, SLOTS - 3] - base).double() * 0.01
-        for slot, name in ((3, "first unit's data arrived"), (4, "first unit's stores issued")):
-            at = start + (d[:, slot] - d[:, 0]).double() * ratio * 1e-3
-            print(f"   on the launch's clock, {name:28s}: p10 {float(at.quantile(.1)):6.2f} us, median {float(at.median()):6.2f}, "
-                  f"p90 {float(at.quantile(.9)):6.2f}, last {float(at.max()):6.2f}")
+    title = (f"rope_rms_kernel, {config} T={T} heads {r.num_heads_q}/{r.num_heads_k}/{r.num_heads_v}, "
+             f"{groups} workgroups x {lanes} lanes, rows stored {'past' if streamed else 'through'} the L2")
+    summarize(buf.cpu(), ROPE_UNIT_PHASES, title)
     assert L.gpuk_stamps_set_rope(None, 0) == 0
-    capi.set_tuning("rope_walk", 0)
 
 
 def main():
@@ -204,7 +174,6 @@ def main():
     rp = sub.add_parser("rope")
     rp.add_argument("--config", choices=["c3", "c4", "c5"], default="c3")
     rp.add_argument("--tokens", type=int, default=0)
-    rp.add_argument("--walk", type=int, default=0, choices=[0, 1, 2], help="0 the launcher's rule, 1 one wave per unit, 2 walking")
     args = ap.parse_args()
     assert torch.cuda.is_available(), "needs a GPU"
     L = bind()
@@ -213,7 +182,7 @@ def main():
             raise SystemExit("static scale: pass a scale through the library's own entry point; not wired here")
         run_norm_quant(L, args.tokens, args.hidden, args.quant)
     else:
-        run_rope(L, args.config, args.tokens, args.walk)
+        run_rope(L, args.config, args.tokens)
 
 
 if __name__ == "__main__":

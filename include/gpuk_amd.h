@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define GPUK_AMD_ABI_VERSION 1
+#define GPUK_AMD_ABI_VERSION 2
 
 typedef enum gpuk_status {
     GPUK_OK = 0,
@@ -198,15 +198,14 @@ int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidden, int dtyp
                                         int *chunks_per_lane);
 
 /*
- * The launch gpuk_rope_rms_set_kv (set_kv != 0) or gpuk_rope_rms (set_kv == 0) makes for a batch with contiguous
- * positions: *walking = 1 for the token-walking kernel (one wave per token or run of tokens), 0 for the kernel with
- * one wave per group of heads; the grid as workgroups x lanes per workgroup; *streamed = 1 when the rotated rows are
- * stored past the L2.  Computed on the host from the sizes and the tuning keys; the four outputs are host pointers.
- * For reports.  Not part of the reference.
+ * The launch gpuk_rope_rms_set_kv (set_kv != 0) or gpuk_rope_rms (set_kv == 0) makes for a batch: the grid as
+ * workgroups x lanes per workgroup (one wave of 64 lanes per group of heads of a token); *streamed = 1 when the
+ * rotated rows are stored past the L2.  Computed on the host from the sizes and the tuning keys; the three outputs
+ * are host pointers.  For reports.  Not part of the reference.
  */
 int gpuk_rope_rms_launch_shape(int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
-                               int64_t head_size, int n_axes, int dtype, int set_kv, int kv_dtype, int *walking,
-                               int *workgroups, int *lanes_per_workgroup, int *streamed);
+                               int64_t head_size, int n_axes, int dtype, int set_kv, int kv_dtype, int *workgroups,
+                               int *lanes_per_workgroup, int *streamed);
 
 /*
  * Launch-cost calibration: data[i] += 1 for i in [0, n) (data 16-byte aligned).  With a small n the call costs
@@ -218,10 +217,9 @@ int gpuk_increment_floats(float *data, int64_t n, void *stream);
 /* Launch-shape knobs for sweeps and for the tests that show the results do not depend on them; value 0 restores
  * the built-in choice.  Keys: "norm_quant_nchunk" (1/2/4/8 16-byte chunks per lane), "norm_quant_threads" (lanes
  * per row), "norm_quant_row_group_shift" (log2 of the run of consecutive rows one XCD takes; -1, not 0, restores the
- * built-in rule), "rope_block_threads" (64/128/256/512, one-wave-per-unit kernel), "rope_walk" (token-walking kernel:
- * 1 never, 2 always), "rope_walk_waves" (waves of its grid), "rope_walk_stream" (output rows of all three rope kernels stored past the L2: 1 never,
- * 2 always), "rope_walk_merge_rows" (1: never fetch an mRoPE token's cos/sin row with one per-lane-addressed
- * transfer).  Unknown keys or values return GPUK_ERR_INVALID_ARG.  The settings are process-global plain variables
+ * built-in rule), "rope_block_threads" (64/128/256/512 lanes per workgroup of the rope kernel), "rope_stream_rows" (output rows of
+ * the rope kernels stored past the L2: 1 never, 2 always), "rope_merge_rows" (1: never let the lanes of an mRoPE
+ * token load their cos/sin pieces straight from the row of their axis).  Unknown keys or values return GPUK_ERR_INVALID_ARG.  The settings are process-global plain variables
  * read at launch: set them from one thread while no other thread is launching.  Not part of the reference. */
 int gpuk_set_tuning(const char *key, int value);
 

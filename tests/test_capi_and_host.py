@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(os.path.join(ROOT, "gpuk_amd", "lib", "libgpuk_amd.so"))
     for n in names:
         assert getattr(lib, n) is not None
-    assert capi.lib().gpuk_abi_version() == 1
+    assert capi.lib().gpuk_abi_version() == 2
     assert capi.lib().gpuk_status_string(0) == b"ok"
     assert b"unsupported" in capi.lib().gpuk_status_string(2)
 
@@ -286,23 +286,21 @@ def test_rope_launch_shape_report():
     """gpuk_rope_rms_launch_shape computes on the host which rope kernel a batch gets, its grid and whether the rotated
     rows are stored past the L2; no GPU is needed."""
     from gpuk_amd import capi
-    # 4096 tokens x (32, 8, 8) heads of 128: one wave per token fills every SIMD four times -> the walking kernel
-    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128) == (True, 1024, 256, False)
-    # in place the kernel with one wave per group of heads is ahead at every size
-    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, set_kv=False) == (False, 5120, 256, True)
-    # three position axes, or an fp8 cache: one wave per group of 8 heads, four waves a workgroup, streamed stores
-    assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3) == (False, 8192, 256, True)
-    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (False, 5120, 256, True)
-    # a decode batch: single waves, through the L2
-    assert capi.rope_rms_launch_shape(16, 28, 4, 4, 128) == (False, 16, 256, False)
-    assert capi.rope_rms_launch_shape(16, 40, 8, 8, 128, kv_fp8=True) == (False, 96, 64, False)
+    # 4096 tokens x (32, 8, 8) heads of 128: one wave per group of 8 Q/K heads, four waves a workgroup, streamed stores
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128) == (5120, 256, True)
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, set_kv=False) == (5120, 256, True)
+    assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3) == (8192, 256, True)
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (5120, 256, True)
+    # a decode batch: through the L2; single waves unless a workgroup of four holds whole tokens
+    assert capi.rope_rms_launch_shape(16, 28, 4, 4, 128) == (16, 256, False)
+    assert capi.rope_rms_launch_shape(16, 40, 8, 8, 128, kv_fp8=True) == (96, 64, False)
     # fp32 activations: a wave per 512/D Q/K heads, and per 512 elements of the V row when a cache is written
-    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32) == (False, 5, 256, True)
-    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32, set_kv=False) == (False, 3, 256, True)
-    assert capi.rope_rms_launch_shape(4, 7, 2, 3, 256, dtype=torch.float64) == (False, 7, 256, True)
+    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32) == (5, 256, True)
+    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32, set_kv=False) == (3, 256, True)
+    assert capi.rope_rms_launch_shape(4, 7, 2, 3, 256, dtype=torch.float64) == (7, 256, True)
     import ctypes as C
     L = capi.lib()
-    o = [C.c_int(0) for _ in range(4)]
+    o = [C.c_int(0) for _ in range(3)]
     refs = [C.byref(x) for x in o]
     assert L.gpuk_rope_rms_launch_shape(0, 32, 8, 8, 128, 1, 0, 1, 0, *refs) == 1
     assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 96, 1, 0, 1, 0, *refs) == 2

@@ -204,7 +204,7 @@ def test_launch_shape_variants(device, threads):
         capi.set_tuning("rope_block_threads", 0)
 
 
-WALK_CASES = [
+HEAD_MIX_CASES = [
     # tokens, (hq, hk, hv), head size, neox, mrope, interleaved, fp8
     (45, (32, 8, 8), 128, True, False, False, False),     # whole units of Q heads, one of K heads
     (61, (28, 4, 4), 128, True, True, False, False),      # a unit that mixes Q and K heads; three position axes
@@ -213,7 +213,7 @@ WALK_CASES = [
     (33, (64, 8, 8), 128, False, False, False, True),     # nine units per token, GPT-J pairs, fp8 cache
     (19, (3, 2, 1), 128, True, False, False, False),      # a single, partly filled unit per token
     (23, (7, 2, 0), 128, True, False, False, False),      # no V heads
-    (41, (28, 4, 4), 128, True, "aligned", False, False),  # sections on multiples of 8: the rows arrive merged
+    (41, (28, 4, 4), 128, True, "aligned", False, False),  # sections on multiples of 8: the lanes load from their axis's row
     (27, (6, 2, 2), 64, False, "aligned", False, True),   # the same with GPT-J pairs, head size 64, fp8 cache
     (31, (36, 0, 8), 128, True, False, False, False),     # no K heads: the last unit holds Q lanes and idle lanes only
     (31, (13, 0, 3), 128, False, False, False, True),     # the same with an fp8 cache, GPT-J pairs
@@ -221,21 +221,18 @@ WALK_CASES = [
     (31, (0, 13, 5), 128, True, False, False, False),     # no Q heads
     (29, (0, 5, 2), 128, False, True, True, True),        # no Q heads, fp8 cache, interleaved sections
 ]
-ALIGNED_SECTIONS = {64: [8, 16, 8], 128: [16, 24, 24], 256: [48, 40, 40]}
 
 
-@pytest.mark.parametrize("case", range(len(WALK_CASES)))
-@pytest.mark.parametrize("waves", [0, 5, 1])
-@pytest.mark.parametrize("stream", [1, 2])
-def test_token_walking_kernel(device, case, waves, stream):
-    """Large batches run a second kernel in which a wave walks the units of whole tokens with the following units'
-    loads in flight.  Forced onto small batches here: as many waves as tokens, five waves, and a single wave that
-    walks every token; stores through the L2 and streamed past it.  Its arithmetic is the one-wave-per-unit
-    kernel's, so besides meeting the oracle the two must agree bit for bit."""
+@pytest.mark.parametrize("case", range(len(HEAD_MIX_CASES)))
+@pytest.mark.parametrize("threads", [0, 64, 512])
+def test_head_mixes_under_both_store_policies(device, case, threads):
+    """Mixes of Q, K and V heads (units of one kind, mixed units, partly filled units, a kind that is absent), padding
+    tokens, text tokens among mRoPE tokens: the oracle's bits with the output rows stored through the L2 and past it,
+    which must also agree with each other bit for bit, whatever the workgroup size."""
     from gpuk_amd import capi
 
-    tokens, heads, hs, neox, mrope, interleaved, fp8 = WALK_CASES[case]
-    print(f"case walk {WALK_CASES[case]} waves={waves} stream={stream}", flush=True)
+    tokens, heads, hs, neox, mrope, interleaved, fp8 = HEAD_MIX_CASES[case]
+    print(f"case head mix {HEAD_MIX_CASES[case]} threads={threads}", flush=True)
     inp = make(tokens, heads[0], hs, neox, seed=900 + case, mrope=bool(mrope), interleaved=interleaved, fp8=fp8, hk=heads[1],
                hv=heads[2])
     if mrope == "aligned":
@@ -243,35 +240,30 @@ def test_token_walking_kernel(device, case, waves, stream):
         inp.positions[:, ::3] = inp.positions[0, ::3]   # every third token a text token: three equal positions
     if case == 0:   # two padding tokens
         inp.kv_loc[3], inp.kv_loc[tokens - 1] = -1, -5
-    nqk = heads[0] + heads[1]
-    capi.set_tuning("rope_walk", 1)
+    capi.set_tuning("rope_block_threads", threads)
     try:
+        capi.set_tuning("rope_stream_rows", 1)
         base_set = run_set_kv(inp, device)
         base_inplace = run_inplace(inp, device)
-        capi.set_tuning("rope_walk", 2)
-        capi.set_tuning("rope_walk_waves", waves)
-        capi.set_tuning("rope_walk_stream", stream)
+        capi.set_tuning("rope_stream_rows", 2)
         got_set = run_set_kv(inp, device)
         got_inplace = run_inplace(inp, device)
     finally:
-        capi.set_tuning("rope_walk", 0)
-        capi.set_tuning("rope_walk_waves", 0)
-        capi.set_tuning("rope_walk_stream", 0)
+        capi.set_tuning("rope_block_threads", 0)
+        capi.set_tuning("rope_stream_rows", 0)
     raw = lambda t: t.cpu().contiguous().view(torch.uint8)
     for name, a, b in zip(("q_out", "k_cache", "v_cache"), got_set[:3], base_set[:3]):
-        assert torch.equal(raw(a), raw(b)), f"{name}: the two kernels differ"
-    assert torch.equal(raw(got_inplace), raw(base_inplace)), "in place: the two kernels differ"
-    check_set_kv(inp, got_set, f"[walk {case}]")
+        assert torch.equal(raw(a), raw(b)), f"{name}: the two store policies differ"
+    assert torch.equal(raw(got_inplace), raw(base_inplace)), "in place: the two store policies differ"
+    check_set_kv(inp, got_set, f"[head mix {case}]")
     check_inplace(inp, got_inplace, "in place")
 
 
-def test_kernel_choice_by_batch_size(device):
-    """The built-in rule: the walking kernel where three or four of its waves sit on nearly every SIMD with one token
-    each (2920-3072 and 3892-4096 tokens), and then only with one position axis, a 16-bit cache and head size 128; the
-    one-wave-per-unit kernel elsewhere, with its q_out / K rows streamed past the L2 from 8 MB per call on.  All of them meet the oracle (sizes
-    on both sides of each switch; mRoPE and plain RoPE; an fp8 cache; too many V heads for the walking kernel)."""
-    cases = ((2900, (32, 8, 8), False, False), (3000, (32, 8, 8), False, False), (4100, (32, 8, 8), False, False),
-             (6100, (12, 4, 4), False, True), (5800, (12, 4, 4), False, True), (4000, (12, 4, 4), True, False),
+def test_batch_sizes_around_the_streaming_rule(device):
+    """Batches below and above the size from which the output rows are stored past the L2 (8 MB per call), with one
+    and three position axes, an fp8 cache, and more V heads than the waves of a token cover in one stride: all of
+    them meet the oracle."""
+    cases = ((3000, (32, 8, 8), False, False), (6100, (12, 4, 4), False, True), (4000, (12, 4, 4), True, False),
              (4000, (12, 4, 4), True, True), (300, (32, 8, 8), False, False), (20100, (4, 4, 10), False, False))
     for tokens, heads, fp8, mrope in cases:
         inp = make(tokens, heads[0], 128, True, seed=tokens, mrope=mrope, fp8=fp8, hk=heads[1], hv=heads[2])
@@ -450,10 +442,9 @@ def test_negative_slots_and_colliding_slots(device, fp8):
     assert bool(k_close.all()), f"K pieces not from any colliding token: {(~k_close).nonzero().flatten().tolist()}"
 
 
-def test_walking_kernel_replayed_from_a_graph(device):
-    """The token-walking kernel (asynchronous global-to-LDS transfers, hand-counted waits) recorded into a HIP graph:
-    every replay, with fresh inputs copied into the captured buffers and eager work in between, equals the eager
-    call on the same inputs."""
+def test_rope_kernel_replayed_from_a_graph(device):
+    """The mRoPE + KV-write op recorded into a HIP graph: every replay, with fresh inputs copied into the captured
+    buffers and eager work in between, equals the eager call on the same inputs."""
     import gpuk_amd as gpuk
     from gpuk_amd import capi
 
@@ -470,7 +461,6 @@ def test_walking_kernel_replayed_from_a_graph(device):
         gpuk.fused_mrope_3d_rms_set_kv(src, qw, kw, cs, positions, T, hq, hk, hv, D, True, inp.mrope_section, False,
                                        inp.eps, q, k, v, loc, 1.0, 1.0)
 
-    capi.set_tuning("rope_walk", 2)
     try:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -496,4 +486,4 @@ def test_walking_kernel_replayed_from_a_graph(device):
             assert torch.equal(raw(q_out), raw(q2)), f"replay {rep}: q_out"
             assert torch.equal(raw(kc[loc]), raw(k2[loc])) and torch.equal(raw(vc[loc]), raw(v2[loc])), f"replay {rep}: cache rows"
     finally:
-        capi.set_tuning("rope_walk", 0)
+        torch.cuda.synchronize()
