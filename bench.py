@@ -293,15 +293,42 @@ def main():
         cp_ms = event_time_ms(lambda i=0: capi.copy_bytes(dst, src, nb), 20)
         extras["copy_kernel_GBps"] = round(2 * nb / (cp_ms * 1e-3) / 1e9, 1)
 
+        def windows(nbytes):
+            """Offsets of windows of nbytes that tile the 512 MiB calibration buffers (at most 16, at least one): calls
+            rotate over them, so that a window comes round again only after the rest of the buffer has passed through
+            the 256 MB last-level cache.  None when not even one window fits."""
+            if nbytes > nb:
+                return None
+            n = max(1, min(16, nb // nbytes))
+            step = (nb - nbytes) // max(n - 1, 1) // 256 * 256 if n > 1 else 0
+            return [k * step for k in range(n)]
+
         def copy_same_bytes_us(nbytes):
             """The plain copy kernel moving as many bytes as a call of a fused kernel moves (half in, half out)."""
             half = (nbytes // 2 + 15) // 16 * 16
-            if half > nb:   # a shape given on the command line whose calls move more than the copy buffers hold
+            offs = windows(half)
+            if offs is None:   # a shape given on the command line whose calls move more than the copy buffers hold
                 return None
-            room = nb - half
-            # three windows of the 512 MiB buffers (the same window three times when only one fits)
-            offs = [((k * half) % room // 256 * 256) if room > 0 else 0 for k in range(3)]
-            return round(event_time_ms(lambda i=0: capi.copy_bytes(dst[offs[i % 3]:], src[offs[i % 3]:], half), 100) * 1e3, 2)
+            n = len(offs)
+            return round(event_time_ms(lambda i=0: capi.copy_bytes(dst[offs[i % n]:], src[offs[i % n]:], half), 100) * 1e3, 2)
+
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+        def one_direction(read_bytes, write_bytes, workgroups, lanes):
+            """What the memory system charges for a call's traffic one direction at a time: a kernel that only reads the
+            call's read bytes, one that only writes its written bytes, and an empty grid of the call's launch shape (the
+            cost of launching and draining it, which each of the two also contains once).  A fused kernel cannot be
+            expected below read + write - launch: reads and writes do not overlap in the memory system."""
+            rb, wb = read_bytes // 16 * 16, write_bytes // 16 * 16
+            ro, wo = windows(rb), windows(wb)
+            if ro is None or wo is None:
+                return None
+            rd = event_time_ms(lambda i=0: capi.read_bytes(src[ro[i % len(ro)]:], rb, sink), 100) * 1e3
+            wr = event_time_ms(lambda i=0: capi.fill_bytes(dst[wo[i % len(wo)]:], wb, i), 100) * 1e3
+            floor = graph_time_us(lambda i=0: capi.empty_grid(workgroups, lanes, 0), 20)
+            return {"read_only_us": round(rd, 2), "read_GBps": round(rb / rd / 1e3, 1), "write_only_us": round(wr, 2),
+                    "write_GBps": round(wb / wr / 1e3, 1), "empty_grid_us": round(floor, 2),
+                    "read_plus_write_minus_launch_us": round(rd + wr - floor, 2)}
 
         # the fused kernel's own memory traffic without its arithmetic (same launch shape, mapping, streaming accesses
         # and barriers) on the benchmark's buffers: the ceiling of the access pattern, beside the kernel itself
@@ -315,7 +342,8 @@ def main():
             "traffic_skeleton_us": round(sk_ms * 1e3, 2), "kernel_us": round(k_ms * 1e3, 2),
             "kernel_over_skeleton": round(k_ms / sk_ms, 4),
             "skeleton_frac_of_8TBps": round(alg_bytes / (sk_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "copy_same_bytes_us": copy_same_bytes_us(alg_bytes)}
+            "copy_same_bytes_us": copy_same_bytes_us(alg_bytes),
+            "one_direction_at_a_time": one_direction(4 * T * H + 2 * H, 3 * T * H + 4 * T, T, lanes)}
 
         def rope_case(r, n_sets):
             n_axes = 3 if r.mrope_section is not None else 1
@@ -338,7 +366,8 @@ def main():
 
             burst = event_time_ms(call, 200)
             avg, med, mn = per_launch_ms(call, 100)
-            return nbytes, avg, med, mn, burst
+            read_bytes = 2 * r.head_size * (r.num_heads_q + r.num_heads_k + r.num_heads_v) * r.num_tokens
+            return nbytes, avg, med, mn, burst, read_bytes
 
         def rope_kernel_label(r):
             # what the launcher picks for this batch, asked of the library
@@ -349,11 +378,15 @@ def main():
                     f"{'past the L2' if streamed else 'through the L2'}")
 
         for name, r in (("rope_kv_qwen3_T4096", workloads.config3()), ("mrope_kv_qwen2vl_T8192", workloads.config4())):
-            nbytes, avg, med, mn, burst = rope_case(r, 4)
+            nbytes, avg, med, mn, burst, read_bytes = rope_case(r, 4)
+            groups, lanes_b, _ = capi.rope_rms_launch_shape(r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v,
+                                                            r.head_size, 3 if r.mrope_section is not None else 1,
+                                                            torch.bfloat16, True, False)
             extras[name] = {"us_per_call": round(burst * 1e3, 2), "avg_launch_us": round(avg * 1e3, 2),
                             "GBps": round(nbytes / (burst * 1e-3) / 1e9, 1),
                             "frac_of_8TBps": round(nbytes / (burst * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                             "algorithmic_bytes": nbytes, "copy_same_bytes_us": copy_same_bytes_us(nbytes),
+                            "one_direction_at_a_time": one_direction(read_bytes, nbytes - read_bytes, groups, lanes_b),
                             "kernel": rope_kernel_label(r)}
         del src, dst
 

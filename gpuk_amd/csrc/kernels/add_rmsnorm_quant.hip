@@ -243,9 +243,10 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
 // is x ^ r and the "codes" fold it to half its size.  What this kernel reaches is the ceiling of the access pattern.
 template <int NCHUNK>
 __global__ void __launch_bounds__(kMaxThreads)
-add_rmsnorm_quant_traffic_only(const u32x4 *x, const u32x4 *residual_in, u32x4 *residual_out, u32x2 *codes,
-                               float *__restrict__ scale_out, int chunks_per_row, int group_shift, int remap_end) {
-    const int tid = threadIdx.x, nthreads = blockDim.x;
+add_rmsnorm_quant_traffic_only(const u32x4 *x, const u32x4 *residual_in, int chunks_per_row, int remap_end,
+                               int group_shift, int nthreads, u32x4 *residual_out, u32x2 *codes,
+                               float *__restrict__ scale_out) {
+    const int tid = threadIdx.x;  // arguments in the order of add_rmsnorm_quant_rows: the same ones arrive in registers
     int row = blockIdx.x;
     if (row < remap_end) {
         const int xcd = row & 7, idx = row >> 3;
@@ -640,10 +641,10 @@ extern "C" int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *re
     auto co = static_cast<u32x2 *>(codes);
     const dim3 grid((unsigned)tokens);
     switch (nchunk) {
-        case 1: add_rmsnorm_quant_traffic_only<1><<<grid, threads, 0, s>>>(xs, rs, ro, co, scale, chunks, group_shift, remap_end); break;
-        case 2: add_rmsnorm_quant_traffic_only<2><<<grid, threads, 0, s>>>(xs, rs, ro, co, scale, chunks, group_shift, remap_end); break;
-        case 4: add_rmsnorm_quant_traffic_only<4><<<grid, threads, 0, s>>>(xs, rs, ro, co, scale, chunks, group_shift, remap_end); break;
-        default: add_rmsnorm_quant_traffic_only<8><<<grid, threads, 0, s>>>(xs, rs, ro, co, scale, chunks, group_shift, remap_end); break;
+        case 1: add_rmsnorm_quant_traffic_only<1><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, group_shift, threads, ro, co, scale); break;
+        case 2: add_rmsnorm_quant_traffic_only<2><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, group_shift, threads, ro, co, scale); break;
+        case 4: add_rmsnorm_quant_traffic_only<4><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, group_shift, threads, ro, co, scale); break;
+        default: add_rmsnorm_quant_traffic_only<8><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, group_shift, threads, ro, co, scale); break;
     }
     return hip_status(hipGetLastError());
 }

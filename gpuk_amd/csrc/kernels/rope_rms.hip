@@ -379,6 +379,9 @@ struct RopeUnit {
 // leave without a round trip for the argument block, which under load costs a wave of this kernel a third of its
 // life; the block (weights, table, outputs, slots) is fetched beside the position, and everything that depends on
 // either is asked for one round trip after entry.  hv_and_waves: hv in bits 0-23, log2 of the waves per workgroup above.
+// (The three-axis instantiations take 66 registers per lane, one wave short of the eight a SIMD can hold; held to 64
+// with amdgpu_waves_per_eu they fit without spilling and run 1-4 % slower: 26.9 against 26.6 us at 8192 tokens of
+// 28+4+4 heads, 51.3 against 49.1 at 16384.)
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 __global__ void __launch_bounds__(512)
 rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_units, uint32_t units_per_token,

@@ -32,14 +32,14 @@ SLOTS = 16   # kStampSlots of csrc/kernels/device_utils.h: 13 clock readings, wa
 STAMPS_LIB = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libgpuk_amd_stamps.so")
 
 NORM_QUANT_PHASES = [
-    (0, 1, "entry -> every load issued (kernel arguments fetched, addresses formed)"),
+    (0, 1, "entry -> every load issued (addresses formed from the arguments the wave finds in its registers)"),
     (1, 2, "-> loads landed (memory latency)"),
     (2, 3, "-> phase 1: residual summed, rounded, stored; the lane's squares summed"),
     (3, 4, "-> sum of squares reduced over the workgroup (DPP, LDS, one barrier)"),
-    (4, 5, "-> rstd (mean, IEEE sqrt and divide)"),
+    (4, 5, "-> rstd (mean, square root and reciprocal, each correctly rounded)"),
     (5, 6, "-> phase 2: row normed (two roundings per element), the lane's maximum"),
     (6, 7, "-> row maximum reduced over the workgroup (DPP, LDS, one barrier)"),
-    (7, 8, "-> scale and its reciprocal (two IEEE divides)"),
+    (7, 8, "-> scale and its reciprocal (two correctly rounded quotients)"),
     (8, 9, "-> phase 3: quotients, fp8 codes, stores issued"),
     (9, 10, "-> every store acknowledged"),
 ]

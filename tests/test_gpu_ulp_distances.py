@@ -34,8 +34,8 @@ def report(name, d, groups_off, group_len):
     return d2 + dmore, worst
 
 
-# beyond-1-ULP element counts measured at these sizes when the bounds were written (kernel A: 0 everywhere)
-NORM_CASES = [("C1 128x4096", lambda: workloads.config1(), 0), ("C2 8192x8192", lambda: workloads.config2(), 0),
+# beyond-1-ULP element counts measured at these sizes when the bounds were written (one element of C2's 67 million)
+NORM_CASES = [("C1 128x4096", lambda: workloads.config1(), 0), ("C2 8192x8192", lambda: workloads.config2(), 1),
               ("C5 512x7168", lambda: workloads.config5_norm(512), 0)]
 
 
@@ -64,8 +64,8 @@ def test_norm_quant_distances_from_the_unmoved_oracle(device, case):
 
 
 # (name, inputs, elements beyond 1 ULP seen in q_out, in the K rows) when the bounds were written
-ROPE_CASES = [("C3", lambda: workloads.config3(), 40, 12), ("C4", lambda: workloads.config4(), 60, 12),
-              ("C5 T=512", lambda: workloads.config5_rope(512), 24, 0)]
+ROPE_CASES = [("C3", lambda: workloads.config3(), 15, 2), ("C4", lambda: workloads.config4(), 37, 1),
+              ("C5 T=512", lambda: workloads.config5_rope(512), 14, 0)]
 
 
 @pytest.mark.parametrize("case", range(len(ROPE_CASES)))
