@@ -61,6 +61,18 @@ __device__ __forceinline__ float div_by_rcp_finite(float a, float b, float rcp) 
     return __builtin_fmaf(-e, rcp, q);
 }
 
+// The codes of one chunk by plain IEEE division, for scales so small or large (or not a number) that a reciprocal
+// leaves the normal range.  Kept out of line: it is long (eight expanded divisions and clamps), it is almost never
+// taken, and inlined it sat between the kernel's last two stretches of common-path code, which a wave then reached
+// by a jump into instructions no prefetch had brought in.
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+__device__ __attribute__((noinline)) u32x2 codes_by_division(f32x8 n, float scale, float fp8_max) {  // by value: in registers
+    float q[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) q[j] = clamp_sym(n[j] / scale, fp8_max);
+    return u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+}
+
 // EXACT: lanes x NCHUNK equals the chunks of a row, so every lane owns NCHUNK live chunks and nothing is masked
 // (true for every power-of-two row and for 7168 elements; it removes a sixth of the kernel's instructions, which is
 // what a decode-sized batch waits for: with at most one row per compute unit the run time is the row's arithmetic).
@@ -206,7 +218,9 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
         // division gives for infinite and NaN numerators.
         constexpr bool kDynamic = QUANT == GPUK_QUANT_FP8_DYNAMIC;
         u32x2 *out = reinterpret_cast<u32x2 *>(norm_out) + row_base;
-        if (__builtin_expect(scale_in_fast_range(scale), 1)) {
+        // (the scale is the same in every lane; deciding by ballot tells the compiler so, and the common path is
+        // laid out as straight-line code with the other one out of the way)
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(!scale_in_fast_range(scale)) == 0, 1)) {
             float rcp;
             if (__builtin_expect(__builtin_amdgcn_ballot_w64(mantissa_all_ones(scale)) == 0, 1)) rcp = rcp_rn_mid_range(scale);
             else rcp = 1.0f / scale;
@@ -221,14 +235,11 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
                 if (live[i]) store_stream(out + i * nthreads + tid, codes);
             }
         } else {
-            // scale so small or large (or not a number) that its reciprocal leaves the normal range: plain IEEE
-            // division (unrolled like the fast path: a runtime index into the register arrays would move them to LDS)
+            // (unrolled like the common path: a runtime index into the register arrays would move them to scratch)
 #pragma unroll
             for (int i = 0; i < NCHUNK; ++i) {
-                float q[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) q[j] = clamp_sym(nv[i][j] / scale, fp8_max);
-                const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                const f32x8 n = {nv[i][0], nv[i][1], nv[i][2], nv[i][3], nv[i][4], nv[i][5], nv[i][6], nv[i][7]};
+                const u32x2 codes = codes_by_division(n, scale, fp8_max);
                 if (live[i]) store_stream(out + i * nthreads + tid, codes);
             }
         }

@@ -420,6 +420,121 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// One wave per token, for batches that the chip holds in one round (one position axis, a cache write, up to
+// kTokenWaveCapacity tokens of UPT units each).  The memory system serves reads and writes one direction at a time,
+// and a kernel of this size (tens of MB each way, 15-20 us) spends a fifth of its time paying for the mix; here the
+// launch is arranged so that there is hardly any: every wave is resident from the start and asks for everything it
+// will read -- all UPT units of its token, its share of nothing but its own token's V row, the weights, then the
+// table row -- before it computes anything, the rotated rows replace the activations in the wave's registers, and
+// no store is issued before `gate` ticks (10 ns) after the wave's entry, the time the launch's reads take at the
+// read-only rate (the host computes it from the bytes of the call).  The chip thus reads for the first half of the
+// launch and writes for the second.  The arithmetic is norm_rotate's, as in the kernel above.
+constexpr uint32_t kTokenWaveCapacity = 4096;  // 4 waves per SIMD: the 100-odd registers a wave of this kernel takes
+// The gate: nine tenths of the time the launch's reads take at 7 TB/s, the rate of a read-only kernel on this part
+// (measured at 2900-4096 tokens of 28+4+4 and 32+8+8 heads: 3-7 % ahead of the kernel above with this gate, 2-4 %
+// with the full time, level or behind with 0.8 or 1.1 times it, and 6 % behind it with no gate at all).
+constexpr double kGateBytesPerTick = 70000.0 / 0.9;
+
+template <typename T, int D, bool NEOX, int UPT, bool KVFP8>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
+rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num_tokens, uint32_t gate, int hq, int hk,
+                      int hv, int64_t ps_token, const RopeArgs rest) {
+    using P = Pack16<T>;
+    constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
+    const uint64_t entry = __builtin_amdgcn_s_memrealtime();
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t t = blockIdx.x * 4 + wave;
+    if (t >= num_tokens) return;
+    const int lane = threadIdx.x & 63, sub = lane % LPH, hl = lane / LPH;
+    const int heads_qk = hq + hk, heads_all = heads_qk + hv, v_chunks = hv * (D / 8);
+    const uint16_t *token_in = static_cast<const uint16_t *>(qkv_in) + (int64_t)t * heads_all * D;
+
+    // ---- everything the wave reads, asked for at once (what needs only the leading parameters first)
+    u32x4 xa[UPT], xb[UPT], v[2];
+#pragma unroll
+    for (int u = 0; u < UPT; ++u) {
+        const int head = min(u * HPW + hl, heads_qk - 1);  // lanes past the last head re-read it
+        const uint16_t *src = token_in + (int64_t)head * D;
+        xa[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 8 * sub));
+        xb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + HALF + 8 * sub));
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int c = min(lane + 64 * j, v_chunks - 1);  // the host admits at most 128 chunks of V per token
+        v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(token_in + (int64_t)heads_qk * D + 8 * c));
+    }
+    const int64_t p0 = positions[(int64_t)t * ps_token];
+    const int64_t slot = rest.kv_loc[t];
+    const uint16_t *qw = static_cast<const uint16_t *>(rest.qw), *kw = static_cast<const uint16_t *>(rest.kw);
+    const u32x4 qwa = *reinterpret_cast<const u32x4 *>(qw + 8 * sub), qwb = *reinterpret_cast<const u32x4 *>(qw + HALF + 8 * sub);
+    const u32x4 kwa = *reinterpret_cast<const u32x4 *>(kw + 8 * sub), kwb = *reinterpret_cast<const u32x4 *>(kw + HALF + 8 * sub);
+    const uint16_t *row = static_cast<const uint16_t *>(rest.cos_sin) + p0 * D;
+    const u32x4 cosv = load_trig<D, NEOX>(row, sub), sinv = load_trig<D, NEOX>(row + HALF, sub);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- norm and rotation, unit by unit, in place
+    const float eps = rest.eps;
+#pragma unroll
+    for (int u = 0; u < UPT; ++u) {
+        const int h0 = u * HPW;
+        u32x4 wa, wb;
+        if (h0 + HPW <= hq) {  // wave-uniform: a unit of Q heads, of K heads, or of both
+            wa = qwa, wb = qwb;
+        } else if (h0 >= hq) {
+            wa = kwa, wb = kwb;
+        } else {
+            const bool is_q = h0 + hl < hq;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wa[j] = is_q ? qwa[j] : kwa[j], wb[j] = is_q ? qwb[j] : kwb[j];
+        }
+        u32x4 oa, ob;
+        norm_rotate<T, D, NEOX>(xa[u], xb[u], wa, wb, cosv, sinv, eps, oa, ob);
+        xa[u] = oa, xb[u] = ob;
+    }
+
+    // ---- the writing half of the launch
+    while (__builtin_amdgcn_s_memrealtime() < entry + gate) __builtin_amdgcn_s_sleep(1);
+    const bool slot_ok = slot >= 0;  // a negative slot: no place in the cache, the K and V rows are dropped
+#pragma unroll
+    for (int u = 0; u < UPT; ++u) {
+        const int head = u * HPW + hl;
+        if (head < hq) {
+            uint16_t *dst = static_cast<uint16_t *>(rest.q_out) + ((int64_t)t * hq + head) * D + 8 * sub;
+            store_pair<HALF * 2>(dst, xa[u], xb[u], true);
+        } else if (head < heads_qk && slot_ok) {
+            const int64_t at = (slot * hk + (head - hq)) * D + 8 * sub;
+            if constexpr (KVFP8) {
+                uint8_t *dst = static_cast<uint8_t *>(rest.k_cache) + at;
+                const float s = rest.k_scale, rcp = 1.0f / s;
+                if (scale_is_fast(s)) {
+                    *reinterpret_cast<u32x2 *>(dst) = quantize_chunk<T, true>(xa[u], s, rcp);
+                    *reinterpret_cast<u32x2 *>(dst + HALF) = quantize_chunk<T, true>(xb[u], s, rcp);
+                } else {
+                    *reinterpret_cast<u32x2 *>(dst) = quantize_chunk<T, false>(xa[u], s, rcp);
+                    *reinterpret_cast<u32x2 *>(dst + HALF) = quantize_chunk<T, false>(xb[u], s, rcp);
+                }
+            } else {
+                store_pair<HALF * 2>(static_cast<uint16_t *>(rest.k_cache) + at, xa[u], xb[u], true);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int c = lane + 64 * j;
+        if (slot_ok && c < v_chunks) {
+            const int64_t off = slot * hv * D + 8 * (int64_t)c;
+            if constexpr (KVFP8) {
+                const float s = rest.v_scale, rcp = 1.0f / s;
+                *reinterpret_cast<u32x2 *>(static_cast<uint8_t *>(rest.v_cache) + off) =
+                    scale_is_fast(s) ? quantize_chunk<T, true>(v[j], s, rcp) : quantize_chunk<T, false>(v[j], s, rcp);
+            } else {
+                *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(rest.v_cache) + off) = v[j];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // fp32 and fp64 activations: the reference dispatches them through the same templates (AT_DISPATCH_FLOATING_TYPES_AND2,
 // src/ops/fused_rope.cpp:27-30, :108-111).  The layout of the 16-bit kernel with chunks of 4 elements: a head is D/8
 // lanes, a lane owns the chunks at elements 4*sub and D/2 + 4*sub of its head (NeoX: x1 and x2 of frequencies
@@ -728,6 +843,9 @@ int launch_2way_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned ba
 int g_block_threads = 0;  // 0 = default
 int g_stream_rows = 0;    // output rows stored past the L2: 0 = built-in rule, 1 = never, 2 = always
 int g_merge_rows = 0;     // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
+int g_token_waves = 0;    // one-wave-per-token kernel: 0 = built-in rule, 1 = never, 2 = wherever it fits
+int g_token_gate = -1;    // its gate in ticks of 10 ns; -1 = from the bytes of the call
+constexpr uint32_t kTokenWaveMinTokens = 2800;
 
 // Streaming stores, measured on MI355X (32/8/8, 28/4/4 and 64/8/8 heads, head sizes 64-256, random slots): q_out /
 // K rows / in-place rows written past the L2 are ahead from about 10 MB per call on (64+8 heads, fp8 cache: 5.9
@@ -739,10 +857,24 @@ constexpr int64_t kStreamFromBytes = 8'000'000;
 struct RopePlan {
     uint32_t threads, blocks;  // workgroup size and count of the launch
     bool stream;               // q_out / K rows / in-place rows stored past the L2
+    bool token_waves;          // the one-wave-per-token kernel
+    uint32_t gate;             // its gate: ticks of 10 ns before which no wave stores
 };
 
-RopePlan plan_rope(const RopeArgs &a, int D, bool set_kv, bool kv_fp8) {
+RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8) {
     RopePlan p{};
+    // One wave per token where the whole batch is resident at once and large enough for its traffic to matter:
+    // one position axis, head size 128, 4 or 5 units (25-40 Q and K heads) and at most 128 chunks of V per token.
+    const int64_t read_bytes = 2 * (int64_t)a.num_tokens * (a.hq + a.hk + a.hv) * D;
+    const bool fits = axes == 1 && set_kv && D == 128 && a.units_per_token >= 4 && a.units_per_token <= 5 &&
+                      a.hv * (D / 8) <= 128 && a.hv > 0 && a.num_tokens <= kTokenWaveCapacity;
+    // ... and where its waves fill the SIMDs evenly, three or four on each: with a SIMD in four holding a wave fewer
+    // the launch waits for the fuller ones (3700 tokens: 1-3 % behind the kernel above; 1024-2048 tokens: level)
+    const uint32_t rounds = (a.num_tokens + 1023) / 1024;
+    const bool even = a.num_tokens >= kTokenWaveMinTokens && 100 * (uint64_t)a.num_tokens >= 94 * (uint64_t)rounds * 1024;
+    p.token_waves = fits && (g_token_waves == 2 || (g_token_waves == 0 && even && !kv_fp8));
+    const double gate = g_token_gate >= 0 ? (double)g_token_gate : (double)read_bytes / kGateBytesPerTick;
+    p.gate = (uint32_t)std::min(gate, 5000.0);
     // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
     const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
     const int64_t call_bytes = set_kv ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
@@ -757,14 +889,34 @@ RopePlan plan_rope(const RopeArgs &a, int D, bool set_kv, bool kv_fp8) {
     p.threads = g_block_threads ? (uint32_t)g_block_threads : (a.units_per_token % 4 == 0 || a.total_units > 8192 ? 256u : 64u);
     const uint32_t units_per_block = p.threads / 64;
     p.blocks = (a.total_units + units_per_block - 1) / units_per_block;
+    if (p.token_waves) {
+        p.threads = 256;
+        p.blocks = (a.num_tokens + 3) / 4;
+        p.stream = true;
+    }
     return p;
 }
 
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
 int launch_one(const RopeArgs &a, hipStream_t stream) {
-    const RopePlan p = plan_rope(a, D, SETKV, KVFP8);
+    const RopePlan p = plan_rope(a, D, AXES, SETKV, KVFP8);
     RopeArgs b = a;
     b.stream_rows = p.stream ? 1u : 0u;
+    if constexpr (AXES == 1 && SETKV && D == 128) {
+        if (p.token_waves) {
+            const uint32_t blocks = (a.num_tokens + 3) / 4;
+#define GPUK_LAUNCH_TOKEN(UPT)                                                                                         \
+    rope_rms_token_kernel<T, D, NEOX, UPT, KVFP8><<<blocks, 256, 0, stream>>>(a.qkv_in, a.positions, a.num_tokens, p.gate,   \
+                                                                            a.hq, a.hk, a.hv, a.ps_token, b)
+            switch (a.units_per_token) {
+                case 4: GPUK_LAUNCH_TOKEN(4); break;
+                case 5: GPUK_LAUNCH_TOKEN(5); break;
+                default: return GPUK_ERR_INTERNAL;
+            }
+#undef GPUK_LAUNCH_TOKEN
+            return hip_status(hipGetLastError());
+        }
+    }
     const uint32_t log2_waves = p.threads == 64 ? 0u : p.threads == 128 ? 1u : p.threads == 256 ? 2u : 3u;
     rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<p.blocks, p.threads, 0, stream>>>(
         a.qkv_in, a.positions, a.total_units, a.units_per_token, a.upt_magic, a.hq, a.hk,
@@ -947,7 +1099,7 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
         *streamed = 1;  // the fp32 / fp64 kernel always stores its rotated rows past the L2
         return GPUK_OK;
     }
-    const RopePlan p = plan_rope(a, (int)D, set_kv, set_kv && kv_dtype == GPUK_KV_E4M3FN);
+    const RopePlan p = plan_rope(a, (int)D, n_axes, set_kv, set_kv && kv_dtype == GPUK_KV_E4M3FN);
     *workgroups = (int)p.blocks;
     *lanes = (int)p.threads;
     *streamed = p.stream ? 1 : 0;
@@ -958,6 +1110,8 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
 
 void set_rope_tuning(int key, int value) {
     if (key == 0) g_block_threads = value;
+    if (key == 1) g_token_waves = value;
+    if (key == 2) g_token_gate = value;
     if (key == 3) g_stream_rows = value;
     if (key == 4) g_merge_rows = value;
 }

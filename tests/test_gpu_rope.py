@@ -259,6 +259,65 @@ def test_head_mixes_under_both_store_policies(device, case, threads):
     check_inplace(inp, got_inplace, "in place")
 
 
+TOKEN_WAVE_CASES = [
+    # tokens, (hq, hk, hv), neox, fp8, fp16
+    (45, (32, 8, 8), True, False, False),     # five units: four of Q heads, one of K heads
+    (61, (28, 4, 4), True, False, False),     # four units, the last one mixes Q and K heads
+    (37, (25, 7, 8), False, True, False),     # a mixed unit in the middle, GPT-J pairs, fp8 cache
+    (31, (36, 0, 8), True, False, False),     # no K heads: the last unit holds Q lanes and idle lanes
+    (29, (0, 33, 5), False, False, False),    # no Q heads, a partly filled last unit, an odd count of V heads
+    (33, (32, 8, 8), False, True, True),      # fp16 activations, fp8 cache
+    (300, (30, 3, 1), True, False, False),    # two rows of waves' worth of workgroups, one V head
+]
+
+
+@pytest.mark.parametrize("case", range(len(TOKEN_WAVE_CASES)))
+@pytest.mark.parametrize("gate", [-1, 0, 700])
+def test_one_wave_per_token_kernel(device, case, gate):
+    """Batches that fit the chip in one round (2800-4096 tokens of 25-40 Q and K heads, one position axis, a cache)
+    run a kernel in which a wave takes a whole token, asks for everything it reads at once and holds its stores back
+    until the launch's reads are through.  Forced onto small batches here, with the gate it would compute, none, and a
+    long one (7 us): the oracle's bits, and the same bits as the kernel with one wave per group of heads."""
+    from gpuk_amd import capi
+
+    tokens, heads, neox, fp8, fp16 = TOKEN_WAVE_CASES[case]
+    print(f"case token waves {TOKEN_WAVE_CASES[case]} gate={gate}", flush=True)
+    inp = make(tokens, heads[0], 128, neox, seed=400 + case, fp8=fp8, hk=heads[1], hv=heads[2])
+    if fp16:
+        inp.qkv, inp.qw, inp.kw, inp.cos_sin = (t.to(torch.float16) for t in (inp.qkv, inp.qw, inp.kw, inp.cos_sin))
+        if not fp8:
+            inp.kv_dtype = torch.float16
+    inp.kv_loc[2], inp.kv_loc[tokens - 1] = -1, -7        # two padding tokens
+    try:
+        capi.set_tuning("rope_token_waves", 1)
+        base = run_set_kv(inp, device)
+        capi.set_tuning("rope_token_waves", 2)
+        capi.set_tuning("rope_token_gate", gate)
+        n_axes = 1
+        groups, lanes, _ = capi.rope_rms_launch_shape(tokens, *heads, 128, n_axes, inp.qkv.dtype, True, fp8)
+        assert (groups, lanes) == ((tokens + 3) // 4, 256), "the case must reach the kernel under test"
+        got = run_set_kv(inp, device)
+    finally:
+        capi.set_tuning("rope_token_waves", 0)
+        capi.set_tuning("rope_token_gate", -1)
+    raw = lambda t: t.cpu().contiguous().view(torch.uint8)
+    for name, a, b in zip(("q_out", "k_cache", "v_cache"), got[:3], base[:3]):
+        assert torch.equal(raw(a), raw(b)), f"{name}: the two kernels differ"
+    check_set_kv(inp, got, f"[token waves {case}]")
+
+
+def test_one_wave_per_token_kernel_by_rule(device):
+    """The launcher's rule takes that kernel where its waves fill the SIMDs evenly, three or four on each (2900 and
+    4000 tokens here), and not in between (3500) or with an fp8 cache; every choice meets the oracle."""
+    from gpuk_amd import capi
+
+    for tokens, fp8, expect in ((2900, False, True), (3500, False, False), (4000, False, True), (4000, True, False)):
+        groups, lanes, _ = capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 1, torch.bfloat16, True, fp8)
+        assert ((groups, lanes) == ((tokens + 3) // 4, 256)) == expect, (tokens, fp8, groups, lanes)
+        inp = make(tokens, 28, 128, True, seed=tokens + 1, fp8=fp8, hk=4, hv=4)
+        check_set_kv(inp, run_set_kv(inp, device), f"[rule T={tokens} fp8={fp8}]")
+
+
 def test_batch_sizes_around_the_streaming_rule(device):
     """Batches below and above the size from which the output rows are stored past the L2 (8 MB per call), with one
     and three position axes, an fp8 cache, and more V heads than the waves of a token cover in one stride: all of
