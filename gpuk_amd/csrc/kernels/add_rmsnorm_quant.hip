@@ -19,6 +19,8 @@
 // 1 KiB (loads) or 512 B (codes) of contiguous memory.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "../../../include/gpuk_amd.h"
 #include "device_utils.h"
 #include "host_utils.h"
@@ -76,20 +78,26 @@ __device__ __attribute__((noinline)) u32x2 codes_by_division(f32x8 n, float scal
 // EXACT: lanes x NCHUNK equals the chunks of a row, so every lane owns NCHUNK live chunks and nothing is masked
 // (true for every power-of-two row and for 7168 elements; it removes a sixth of the kernel's instructions, which is
 // what a decode-sized batch waits for: with at most one row per compute unit the run time is the row's arithmetic).
-template <typename T, int NCHUNK, int QUANT, bool EXACT>
+template <typename T, int NCHUNK, int QUANT, bool EXACT, bool GATED>
 __global__ void __launch_bounds__(kMaxThreads)
-add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_row, int remap_end, int group_shift,
-                       int nthreads, const u32x4 *__restrict__ gamma, u32x4 *residual_out, void *norm_out,
-                       float *__restrict__ scale_io, float hidden_f, float rcp_hidden, int hidden_pow2, float eps,
-                       float fp8_max, float rcp_fp8_max) {
+add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_row, int remap_end,
+                       uint32_t lanes_and_shift, uint32_t gate, const u32x4 *__restrict__ gamma, u32x4 *residual_out,
+                       void *norm_out, float *__restrict__ scale_io, float hidden_f, float rcp_hidden, int hidden_pow2,
+                       float eps, float fp8_max, float rcp_fp8_max) {
     // The arguments are ordered by when a wave needs them: the first fourteen dwords (up to norm_out) are handed to
     // the wave in scalar registers at launch (-amdgpu-kernarg-preload-count), so the loads of the row are issued
-    // without a round trip for the argument block; nthreads is the workgroup size, passed so that it need not be
-    // fetched from the dispatch packet either.
+    // without a round trip for the argument block; lanes_and_shift holds the workgroup size (bits 0-15), passed so
+    // that it need not be fetched from the dispatch packet either, and the row-run shift (bits 16-31).
+    const int nthreads = (int)(lanes_and_shift & 0xffffu), group_shift = (int)(lanes_and_shift >> 16);
     using P = Pack16<T>;
     __shared__ float s_sum[kReduceSlots];
     __shared__ float s_max[kReduceSlots];
     GPUK_STAMPS_BEGIN();  // profiling build only
+    // GATED (batches whose rows are all resident at once): no store before `gate` ticks of 10 ns after the wave's
+    // entry, the time the launch's reads take; the chip then reads in the first part of the launch and writes in the
+    // second instead of mixing the two, which the memory system charges for.  The residual is stored with the codes.
+    // (A template parameter: as a run-time choice the branches around the early stores cost the large batches 1 %.)
+    const uint64_t entry = GATED ? __builtin_amdgcn_s_memrealtime() : 0;
 
     const int tid = threadIdx.x;
     const int num_waves = nthreads >> 6;
@@ -140,7 +148,7 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
             if (j & 1) ss1 = P::add_squares(w, ss1);
             else ss0 = P::add_squares(w, ss0);
         }
-        if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+        if (!GATED && live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
     }
     float sumsq[1] = {ss0 + ss1};
     GPUK_STAMP(3);  // residual stored, the lane's squares summed
@@ -161,15 +169,25 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
     GPUK_STAMP(5);  // rstd
     if constexpr (QUANT == GPUK_QUANT_NONE) {
         u32x4 *out = reinterpret_cast<u32x4 *>(norm_out) + row_base;
+        u32x4 normed[NCHUNK];
 #pragma unroll
         for (int i = 0; i < NCHUNK; ++i) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const float lo = P::lo(gv[i][j]) * P::round(P::lo(xv[i][j]) * rstd);
                 const float hi = P::hi(gv[i][j]) * P::round(P::hi(xv[i][j]) * rstd);
-                xv[i][j] = P::pack(lo, hi);  // xv now holds the normed row
+                normed[i][j] = P::pack(lo, hi);
             }
-            if (live[i]) store_stream(out + i * nthreads + tid, xv[i]);
+            if (!GATED && live[i]) store_stream(out + i * nthreads + tid, normed[i]);
+        }
+        if constexpr (GATED) {
+            while (__builtin_amdgcn_s_memrealtime() < entry + gate) __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i)
+                if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i)
+                if (live[i]) store_stream(out + i * nthreads + tid, normed[i]);
         }
         GPUK_STAMP(9);
         GPUK_STAMP_DRAINED(10);
@@ -225,16 +243,31 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
             if (__builtin_expect(__builtin_amdgcn_ballot_w64(mantissa_all_ones(scale)) == 0, 1)) rcp = rcp_rn_mid_range(scale);
             else rcp = 1.0f / scale;
             GPUK_STAMP(8);  // scale and its reciprocal
+            u32x2 codes[NCHUNK];
 #pragma unroll
             for (int i = 0; i < NCHUNK; ++i) {
                 float q[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) q[j] = kDynamic ? div_by_rcp_finite(nv[i][j], scale, rcp) : div_by_rcp(nv[i][j], scale, rcp);
                 if constexpr (!kDynamic) clamp8_sym(q, fp8_max);
-                const u32x2 codes = {cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
-                if (live[i]) store_stream(out + i * nthreads + tid, codes);
+                codes[i] = u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
+                if (!GATED && live[i]) store_stream(out + i * nthreads + tid, codes[i]);
+            }
+            if constexpr (GATED) {
+                while (__builtin_amdgcn_s_memrealtime() < entry + gate) __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+                for (int i = 0; i < NCHUNK; ++i)
+                    if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+#pragma unroll
+                for (int i = 0; i < NCHUNK; ++i)
+                    if (live[i]) store_stream(out + i * nthreads + tid, codes[i]);
             }
         } else {
+            if constexpr (GATED) {  // (no wait on this path: it is taken by rows whose scale is degenerate)
+#pragma unroll
+                for (int i = 0; i < NCHUNK; ++i)
+                    if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+            }
             // (unrolled like the common path: a runtime index into the register arrays would move them to scratch)
 #pragma unroll
             for (int i = 0; i < NCHUNK; ++i) {
@@ -255,8 +288,10 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
 template <int NCHUNK>
 __global__ void __launch_bounds__(kMaxThreads)
 add_rmsnorm_quant_traffic_only(const u32x4 *x, const u32x4 *residual_in, int chunks_per_row, int remap_end,
-                               int group_shift, int nthreads, u32x4 *residual_out, u32x2 *codes,
+                               uint32_t lanes_and_shift, uint32_t gate, u32x4 *residual_out, u32x2 *codes,
                                float *__restrict__ scale_out) {
+    const int nthreads = (int)(lanes_and_shift & 0xffffu), group_shift = (int)(lanes_and_shift >> 16);
+    const uint64_t entry = __builtin_amdgcn_s_memrealtime();  // the kernel's store gate, see there
     const int tid = threadIdx.x;  // arguments in the order of add_rmsnorm_quant_rows: the same ones arrive in registers
     int row = blockIdx.x;
     if (row < remap_end) {
@@ -276,10 +311,16 @@ add_rmsnorm_quant_traffic_only(const u32x4 *x, const u32x4 *residual_in, int chu
 #pragma unroll
     for (int i = 0; i < NCHUNK; ++i) {
         xv[i] ^= rv[i];
-        if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+        if (!gate && live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
     }
     __syncthreads();
     __syncthreads();
+    if (gate) {
+        while (__builtin_amdgcn_s_memrealtime() < entry + gate) __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+        for (int i = 0; i < NCHUNK; ++i)
+            if (live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
+    }
     if (tid == 0) scale_out[row] = 1.0f;
 #pragma unroll
     for (int i = 0; i < NCHUNK; ++i) {
@@ -474,6 +515,23 @@ add_rmsnorm_quant_wide_rows(const wide4<F> *x, const wide4<F> *residual_in,  // 
 int g_force_nchunk = 0;   // 0 = heuristic; set through gpuk_set_tuning for sweeps
 int g_force_threads = 0;  // 0 = heuristic
 int g_row_group_shift = -1;  // -1 = heuristic, else log2 of the run of consecutive rows an XCD takes (0 = one row)
+int g_gate = -1;             // store gate in ticks of 10 ns: -1 = built-in rule, 0 = none, > 0 = that many
+constexpr int kComputeUnits = 256;  // MI355X
+
+// The store gate of a launch of 16-bit rows: for batches whose workgroups are all resident at once (2048 lanes per
+// compute unit) the time their reads take at 7 TB/s, the rate of a read-only kernel on this part, plus a twentieth;
+// 0 (stores as soon as they are ready) for larger batches, whose later workgroups read while earlier ones write
+// whatever a wave does.  Measured per call at 7168 elements: 6.35 against 7.2 us at 512 rows, 7.6 against 9.5 at
+// 768, 9.0 against 11.7 at 1024 (gate 1.0-1.1 times the read time; 10.2 with 0.9, 9.6 with 1.2), nothing gained and
+// 0.1 us lost below a quarter of a round; at 4096 elements 6.2 against 7.7 us at 1024 rows, 10.2 against 12.4 at 2048; 20-45 % slower where the
+// batch does not fit one round.
+uint32_t store_gate(int64_t tokens, int64_t hidden, int threads) {
+    if (g_gate >= 0) return (uint32_t)g_gate;
+    const int64_t resident_rows = (int64_t)kComputeUnits * (2048 / threads);
+    if (tokens > resident_rows || 4 * tokens < resident_rows) return 0;
+    const double ticks = 1.05 * (double)(4 * tokens * hidden) / 70000.0;  // 70,000 bytes per tick of 10 ns
+    return (uint32_t)std::min(ticks, 5000.0);
+}
 
 // Lanes per row and chunks per lane.  Measured on MI355X over rows of 1024 .. 16384 elements: two chunks per lane
 // on as many lanes as that needs (up to 1024) streams best or ties everywhere (1-6 % over one or four chunks per
@@ -523,6 +581,7 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
     const float rcp_hidden = 1.0f / hf;
     const int hidden_pow2 = (hidden & (hidden - 1)) == 0;
     const float rcp_fp8_max = (fp8_max == 448.0f || fp8_max == 240.0f) ? 1.0f / fp8_max : 0.0f;
+    const uint32_t gate = store_gate(tokens, hidden, threads);
     // Runs of 64 rows per XCD: measured +1.1 % for 16 KiB rows (8192 rows); neutral or 1-10 % slower for every other
     // row size tried (2, 3, 4, 8, 10, 14, 32 KiB) and for fewer rows, hence the narrow rule.
     const int64_t row_bytes = hidden * 2;
@@ -530,14 +589,16 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
     if (g_row_group_shift >= 0) group_shift = g_row_group_shift;
     const int remap_end = group_shift > 0 ? (int)((tokens >> (3 + group_shift)) << (3 + group_shift)) : 0;
     const bool exact = (int64_t)threads * nchunk == chunks;
+#define GPUK_LAUNCH_NQ_AS(N, EXACT, GATED)                                                                              \
+    add_rmsnorm_quant_rows<T, N, QUANT, EXACT, GATED><<<grid, threads, 0, stream>>>(                                    \
+        xs, rs, chunks, remap_end, (uint32_t)threads | ((uint32_t)group_shift << 16), gate, gs, ro, norm_out, scale, hf, \
+        rcp_hidden, hidden_pow2, eps, fp8_max, rcp_fp8_max)
 #define GPUK_LAUNCH_NQ(N)                                                                                              \
     do {                                                                                                               \
-        if (exact)                                                                                                     \
-            add_rmsnorm_quant_rows<T, N, QUANT, true><<<grid, threads, 0, stream>>>(                                   \
-                xs, rs, chunks, remap_end, group_shift, threads, gs, ro, norm_out, scale, hf, rcp_hidden, hidden_pow2, eps, fp8_max, rcp_fp8_max); \
-        else                                                                                                           \
-            add_rmsnorm_quant_rows<T, N, QUANT, false><<<grid, threads, 0, stream>>>(                                  \
-                xs, rs, chunks, remap_end, group_shift, threads, gs, ro, norm_out, scale, hf, rcp_hidden, hidden_pow2, eps, fp8_max, rcp_fp8_max); \
+        if (exact && gate) GPUK_LAUNCH_NQ_AS(N, true, true);                                                           \
+        else if (exact) GPUK_LAUNCH_NQ_AS(N, true, false);                                                             \
+        else if (gate) GPUK_LAUNCH_NQ_AS(N, false, true);                                                              \
+        else GPUK_LAUNCH_NQ_AS(N, false, false);                                                                       \
     } while (0)
     switch (nchunk) {
         case 1: GPUK_LAUNCH_NQ(1); break;
@@ -547,6 +608,7 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
         default: return GPUK_ERR_INTERNAL;
     }
 #undef GPUK_LAUNCH_NQ
+#undef GPUK_LAUNCH_NQ_AS
     return hip_status(hipGetLastError());
 }
 
@@ -625,6 +687,7 @@ void set_norm_quant_tuning(int key, int value) {
     if (key == 0) g_force_nchunk = value;
     if (key == 1) g_force_threads = value;
     if (key == 5) g_row_group_shift = value;
+    if (key == 6) g_gate = value;
 }
 
 }  // namespace gpuk
@@ -651,11 +714,13 @@ extern "C" int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *re
     auto ro = static_cast<u32x4 *>(residual_out);
     auto co = static_cast<u32x2 *>(codes);
     const dim3 grid((unsigned)tokens);
+    const uint32_t gate = store_gate(tokens, hidden, threads);
+    const uint32_t shape = (uint32_t)threads | ((uint32_t)group_shift << 16);
     switch (nchunk) {
-        case 1: add_rmsnorm_quant_traffic_only<1><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, group_shift, threads, ro, co, scale); break;
-        case 2: add_rmsnorm_quant_traffic_only<2><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, group_shift, threads, ro, co, scale); break;
-        case 4: add_rmsnorm_quant_traffic_only<4><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, group_shift, threads, ro, co, scale); break;
-        default: add_rmsnorm_quant_traffic_only<8><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, group_shift, threads, ro, co, scale); break;
+        case 1: add_rmsnorm_quant_traffic_only<1><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, shape, gate, ro, co, scale); break;
+        case 2: add_rmsnorm_quant_traffic_only<2><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, shape, gate, ro, co, scale); break;
+        case 4: add_rmsnorm_quant_traffic_only<4><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, shape, gate, ro, co, scale); break;
+        default: add_rmsnorm_quant_traffic_only<8><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, shape, gate, ro, co, scale); break;
     }
     return hip_status(hipGetLastError());
 }

@@ -439,7 +439,6 @@ template <typename T, int D, bool NEOX, int UPT, bool KVFP8>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
 rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num_tokens, uint32_t gate, int hq, int hk,
                       int hv, int64_t ps_token, const RopeArgs rest) {
-    using P = Pack16<T>;
     constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
     const uint64_t entry = __builtin_amdgcn_s_memrealtime();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);

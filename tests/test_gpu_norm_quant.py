@@ -195,6 +195,26 @@ def test_launch_shape_variants(device, threads, nchunk):
         capi.set_tuning("norm_quant_threads", 0)
 
 
+@pytest.mark.parametrize("gate", [0, 1, 300])
+def test_store_gate_changes_no_bits(device, gate):
+    """Batches whose workgroups are all resident at once hold their stores back until the launch's reads are through
+    (the residual is then stored with the codes); larger ones store as soon as they can.  Both orders, forced onto
+    the same small batch -- no gate, the shortest one and 3 us -- give the oracle's bits in every quant mode."""
+    from gpuk_amd import capi
+
+    print(f"case store gate {gate}", flush=True)
+    capi.set_tuning("norm_quant_gate", gate)
+    try:
+        for tokens, hidden in ((300, 7168), (64, 4096), (5, 1032)):
+            inp = workloads.norm_quant_inputs(tokens, hidden, seed=gate + hidden, res_sigma=2.0, outlier_frac=0.01)
+            for quant in (0, 1, 3):
+                st = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
+                check(inp, quant, run_capi(inp, quant, device, static_scale=st), static_scale=st,
+                      tag=f"[gate {gate} {tokens}x{hidden} q{quant}]")
+    finally:
+        capi.set_tuning("norm_quant_gate", -1)
+
+
 @pytest.mark.parametrize("alias", ["residual_in", "x"])
 @pytest.mark.parametrize("quant", [0, 1, 3])
 def test_residual_out_may_alias_an_input(device, alias, quant):
