@@ -371,15 +371,16 @@ def main():
 
         def rope_kernel_label(r):
             # what the launcher picks for this batch, asked of the library
-            groups, lanes, streamed = capi.rope_rms_launch_shape(
+            groups, lanes, streamed, token_waves = capi.rope_rms_launch_shape(
                 r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
                 3 if r.mrope_section is not None else 1, torch.bfloat16, True, r.kv_dtype == torch.float8_e4m3fn)
-            return (f"rope_rms_kernel (one wave per group of heads), {groups} workgroups x {lanes} lanes, rows stored "
-                    f"{'past the L2' if streamed else 'through the L2'}")
+            form = ("rope_rms_token_kernel (one wave per token, stores gated behind the launch's reads)" if token_waves
+                    else "rope_rms_kernel (one wave per group of heads)")
+            return f"{form}, {groups} workgroups x {lanes} lanes, rows stored {'past the L2' if streamed else 'through the L2'}"
 
         for name, r in (("rope_kv_qwen3_T4096", workloads.config3()), ("mrope_kv_qwen2vl_T8192", workloads.config4())):
             nbytes, avg, med, mn, burst, read_bytes = rope_case(r, 4)
-            groups, lanes_b, _ = capi.rope_rms_launch_shape(r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v,
+            groups, lanes_b, _, _ = capi.rope_rms_launch_shape(r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v,
                                                             r.head_size, 3 if r.mrope_section is not None else 1,
                                                             torch.bfloat16, True, False)
             extras[name] = {"us_per_call": round(burst * 1e3, 2), "avg_launch_us": round(avg * 1e3, 2),

@@ -55,6 +55,7 @@ struct RopeArgs {
     uint32_t num_tokens;
     uint32_t stream_rows;  // 1: q_out / K rows / in-place rows are stored past the L2 (calls that move more than a few MB)
     uint32_t merge_rows;   // mRoPE: every aligned group of 8 frequencies takes one axis: each lane loads from that axis's row
+    uint32_t gate;         // ticks of 10 ns after a wave's entry before which it stores nothing (0 = no gate)
 };
 
 // dword mask selecting the 16-bit halves whose bit is set in a 2-bit field
@@ -316,8 +317,10 @@ struct RopeUnit {
         }
     }
 
-    // Norm, rotation and all stores of the unit.
-    static __device__ __forceinline__ void finish(const RopeArgs &a, int lane, UnitState &st) {
+    // Norm, rotation and all stores of the unit.  GATED: no store before a.gate ticks after `entry`, the wave's entry
+    // time (a template parameter: as a run-time choice the check cost the launches without a gate 2-6 %).
+    template <bool GATED>
+    static __device__ __forceinline__ void finish(const RopeArgs &a, int lane, UnitState &st, uint64_t entry) {
         if (!st.live) return;
         const int sub = lane % LPH;
         const int heads_qk = a.hq + a.hk, heads_all = heads_qk + a.hv;
@@ -325,6 +328,8 @@ struct RopeUnit {
 
         u32x4 oa, ob;
         norm_rotate<T, D, NEOX>(xa, xb, wa, wb, cosv, sinv, a.eps, oa, ob);
+        // batches whose waves are all resident at once: no store before the launch's reads are through
+        if constexpr (GATED) while (__builtin_amdgcn_s_memrealtime() < entry + a.gate) __builtin_amdgcn_s_sleep(1);
 
         // A negative slot marks a token that has no place in the cache (padding in a fixed-size decode batch): its Q
         // row is still produced, its K and V rows are dropped.  The reference would write out of bounds.
@@ -382,7 +387,7 @@ struct RopeUnit {
 // (The three-axis instantiations take 66 registers per lane, one wave short of the eight a SIMD can hold; held to 64
 // with amdgpu_waves_per_eu they fit without spilling and run 1-4 % slower: 26.9 against 26.6 us at 8192 tokens of
 // 28+4+4 heads, 51.3 against 49.1 at 16384.)
-template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8>
+template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8, bool GATED>
 __global__ void __launch_bounds__(512)
 rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_units, uint32_t units_per_token,
                 uint32_t upt_magic, int hq, int hk, uint32_t hv_and_waves, int64_t ps_token, int64_t ps_axis,
@@ -391,6 +396,7 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t unit = (blockIdx.x << (hv_and_waves >> 24)) + wave;
     if (unit >= total_units) return;
+    const uint64_t entry = GATED ? __builtin_amdgcn_s_memrealtime() : 0;
     RopeArgs a = rest;  // the fields that came ahead replace their copies in the block
     a.qkv_in = qkv_in;
     a.positions = positions;
@@ -413,7 +419,7 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
     // moves arithmetic above later loads and the wave pays several memory round trips in a row.
     __builtin_amdgcn_sched_barrier(0);
     GPUK_STAMP_DRAINED(3);  // everything landed
-    Unit::finish(a, lane, st);
+    Unit::template finish<GATED>(a, lane, st, entry);
     GPUK_STAMP(4);          // rows stored (issued)
     GPUK_STAMP_DRAINED(5);  // ... and acknowledged
     GPUK_STAMPS_WRITE(unit);
@@ -844,6 +850,7 @@ int g_stream_rows = 0;    // output rows stored past the L2: 0 = built-in rule, 
 int g_merge_rows = 0;     // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
 int g_token_waves = 0;    // one-wave-per-token kernel: 0 = built-in rule, 1 = never, 2 = wherever it fits
 int g_token_gate = -1;    // its gate in ticks of 10 ns; -1 = from the bytes of the call
+int g_unit_gate = -1;     // gate of the kernel with one wave per unit: -1 = built-in rule, 0 = none, > 0 = ticks
 constexpr uint32_t kTokenWaveMinTokens = 2800;
 
 // Streaming stores, measured on MI355X (32/8/8, 28/4/4 and 64/8/8 heads, head sizes 64-256, random slots): q_out /
@@ -858,6 +865,7 @@ struct RopePlan {
     bool stream;               // q_out / K rows / in-place rows stored past the L2
     bool token_waves;          // the one-wave-per-token kernel
     uint32_t gate;             // its gate: ticks of 10 ns before which no wave stores
+    uint32_t unit_gate;        // the same for the kernel with one wave per unit (0 = none)
 };
 
 RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8) {
@@ -874,6 +882,16 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     p.token_waves = fits && (g_token_waves == 2 || (g_token_waves == 0 && even && !kv_fp8));
     const double gate = g_token_gate >= 0 ? (double)g_token_gate : (double)read_bytes / kGateBytesPerTick;
     p.gate = (uint32_t)std::min(gate, 5000.0);
+    // The kernel with one wave per unit gates its stores in the same way where its waves are all resident at once
+    // (8192 of them, eight per SIMD, with one position axis) and fill at least half of that round; the gate is the
+    // read time at 7 TB/s.  Measured with a cache write: 64+8+8 heads, fp8 cache, 7.7 against 8.5 us at 768 tokens, 8.6
+    // against 9.5 at 900; 32+8+8 heads 6.1 against 7.0 us at 1024 tokens, 8.4 against 9.5 at 1600; nothing to gain
+    // below half a round, 15-35 % slower one unit beyond it (10.4 -> 11.9 us at 1024 tokens of 64+8+8 heads), and
+    // 2 % at best with three position axes, whose instantiations hold seven waves per SIMD.
+    p.unit_gate = 0;
+    if (g_unit_gate > 0) p.unit_gate = (uint32_t)g_unit_gate;
+    else if (g_unit_gate < 0 && axes == 1 && set_kv && a.total_units <= 8192 && a.total_units >= 4096)
+        p.unit_gate = (uint32_t)std::min((double)read_bytes / 70000.0, 5000.0);
     // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
     const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
     const int64_t call_bytes = set_kv ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
@@ -901,6 +919,7 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
     const RopePlan p = plan_rope(a, D, AXES, SETKV, KVFP8);
     RopeArgs b = a;
     b.stream_rows = p.stream ? 1u : 0u;
+    b.gate = p.unit_gate;
     if constexpr (AXES == 1 && SETKV && D == 128) {
         if (p.token_waves) {
             const uint32_t blocks = (a.num_tokens + 3) / 4;
@@ -917,9 +936,18 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
         }
     }
     const uint32_t log2_waves = p.threads == 64 ? 0u : p.threads == 128 ? 1u : p.threads == 256 ? 2u : 3u;
-    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8><<<p.blocks, p.threads, 0, stream>>>(
-        a.qkv_in, a.positions, a.total_units, a.units_per_token, a.upt_magic, a.hq, a.hk,
-        (uint32_t)a.hv | (log2_waves << 24), a.ps_token, a.ps_axis, b);
+#define GPUK_LAUNCH_UNITS(GATED)                                                                                        \
+    rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8, GATED><<<p.blocks, p.threads, 0, stream>>>(                         \
+        a.qkv_in, a.positions, a.total_units, a.units_per_token, a.upt_magic, a.hq, a.hk,                               \
+        (uint32_t)a.hv | (log2_waves << 24), a.ps_token, a.ps_axis, b)
+    if constexpr (AXES == 1 && SETKV) {  // the only launches the rule gates
+        if (b.gate) GPUK_LAUNCH_UNITS(true);
+        else GPUK_LAUNCH_UNITS(false);
+    } else {
+        b.gate = 0;
+        GPUK_LAUNCH_UNITS(false);
+    }
+#undef GPUK_LAUNCH_UNITS
     return hip_status(hipGetLastError());
 }
 
@@ -1076,10 +1104,11 @@ int rope_common(const void *qkv_in, void *qkv_out, const void *qw, const void *k
 }
 
 int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, int n_axes, int dtype, bool set_kv,
-                      int kv_dtype, int *workgroups, int *lanes, int *streamed) {
+                      int kv_dtype, int *workgroups, int *lanes, int *streamed, int *token_waves) {
     if (T <= 0 || hq < 0 || hk < 0 || hv < 0 || hq + hk == 0 || (n_axes != 1 && n_axes != 3)) return GPUK_ERR_INVALID_ARG;
     if (D != 64 && D != 128 && D != 256) return GPUK_ERR_UNSUPPORTED;
-    if (!workgroups || !lanes || !streamed) return GPUK_ERR_INVALID_ARG;
+    if (!workgroups || !lanes || !streamed || !token_waves) return GPUK_ERR_INVALID_ARG;
+    *token_waves = 0;
     if (dtype != GPUK_DTYPE_BF16 && dtype != GPUK_DTYPE_FP16 && dtype != GPUK_DTYPE_F32 && dtype != GPUK_DTYPE_F64) return GPUK_ERR_UNSUPPORTED;
     const bool wide = dtype == GPUK_DTYPE_F32 || dtype == GPUK_DTYPE_F64;
     const int64_t hpw = 64 / (D / 16);
@@ -1102,6 +1131,7 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
     *workgroups = (int)p.blocks;
     *lanes = (int)p.threads;
     *streamed = p.stream ? 1 : 0;
+    *token_waves = p.token_waves ? 1 : 0;
     return GPUK_OK;
 }
 
@@ -1109,6 +1139,7 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
 
 void set_rope_tuning(int key, int value) {
     if (key == 0) g_block_threads = value;
+    if (key == 6) g_unit_gate = value;
     if (key == 1) g_token_waves = value;
     if (key == 2) g_token_gate = value;
     if (key == 3) g_stream_rows = value;
@@ -1123,9 +1154,9 @@ GPUK_STAMPS_SETTER(gpuk_stamps_set_rope)
 extern "C" int gpuk_rope_rms_launch_shape(int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k,
                                           int64_t num_heads_v, int64_t head_size, int n_axes, int dtype, int set_kv,
                                           int kv_dtype, int *workgroups, int *lanes_per_workgroup,
-                                          int *streamed) {
+                                          int *streamed, int *token_waves) {
     return gpuk::rope_launch_shape(num_tokens, num_heads_q, num_heads_k, num_heads_v, head_size, n_axes, dtype,
-                                   set_kv != 0, kv_dtype, workgroups, lanes_per_workgroup, streamed);
+                                   set_kv != 0, kv_dtype, workgroups, lanes_per_workgroup, streamed, token_waves);
 }
 
 extern "C" int gpuk_rope_rms(void *qkv, const void *qw, const void *kw, const void *cos_sin, const int64_t *positions,

@@ -140,7 +140,8 @@ def run_rope(L, config, tokens):
         r = workloads.config5_rope(tokens or 128)
     T = r.num_tokens
     n_axes = 3 if r.mrope_section is not None else 1
-    groups, lanes, streamed = capi.rope_rms_launch_shape(T, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
+    capi.set_tuning("rope_token_waves", 1)   # the stamps are in the kernel with one wave per group of heads
+    groups, lanes, streamed, _ = capi.rope_rms_launch_shape(T, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
                                                                   n_axes, torch.bfloat16, True, r.kv_dtype == torch.float8_e4m3fn)
     waves = groups * (lanes // 64)
     buf = torch.zeros((waves, SLOTS), dtype=torch.int64, device=dev)
@@ -162,6 +163,7 @@ def run_rope(L, config, tokens):
              f"{groups} workgroups x {lanes} lanes, rows stored {'past' if streamed else 'through'} the L2")
     summarize(buf.cpu(), ROPE_UNIT_PHASES, title)
     assert L.gpuk_stamps_set_rope(None, 0) == 0
+    capi.set_tuning("rope_token_waves", 0)
 
 
 def main():

@@ -199,13 +199,14 @@ int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidden, int dtyp
 
 /*
  * The launch gpuk_rope_rms_set_kv (set_kv != 0) or gpuk_rope_rms (set_kv == 0) makes for a batch: the grid as
- * workgroups x lanes per workgroup (one wave of 64 lanes per group of heads of a token); *streamed = 1 when the
- * rotated rows are stored past the L2.  Computed on the host from the sizes and the tuning keys; the three outputs
- * are host pointers.  For reports.  Not part of the reference.
+ * workgroups x lanes per workgroup; *streamed = 1 when the rotated rows are stored past the L2; *token_waves = 1 for
+ * the kernel in which a wave of 64 lanes takes a whole token (batches the chip holds in one round), 0 for the one in
+ * which it takes a group of heads of a token.  Computed on the host from the sizes and the tuning keys; the four
+ * outputs are host pointers.  For reports.  Not part of the reference.
  */
 int gpuk_rope_rms_launch_shape(int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
                                int64_t head_size, int n_axes, int dtype, int set_kv, int kv_dtype, int *workgroups,
-                               int *lanes_per_workgroup, int *streamed);
+                               int *lanes_per_workgroup, int *streamed, int *token_waves);
 
 /*
  * Launch-cost calibration: data[i] += 1 for i in [0, n) (data 16-byte aligned).  With a small n the call costs

@@ -287,22 +287,22 @@ def test_rope_launch_shape_report():
     rows are stored past the L2; no GPU is needed."""
     from gpuk_amd import capi
     # 4096 tokens x (32, 8, 8) heads of 128 with a 16-bit cache: the batch fits the chip in one round, one wave per token
-    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128) == (1024, 256, True)
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128) == (1024, 256, True, True)
     # 4200 tokens do not: one wave per group of 8 Q/K heads, four waves a workgroup, streamed stores
-    assert capi.rope_rms_launch_shape(4200, 32, 8, 8, 128) == (5250, 256, True)
-    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, set_kv=False) == (5120, 256, True)
-    assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3) == (8192, 256, True)
-    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (5120, 256, True)
+    assert capi.rope_rms_launch_shape(4200, 32, 8, 8, 128) == (5250, 256, True, False)
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, set_kv=False) == (5120, 256, True, False)
+    assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3) == (8192, 256, True, False)
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (5120, 256, True, False)
     # a decode batch: through the L2; single waves unless a workgroup of four holds whole tokens
-    assert capi.rope_rms_launch_shape(16, 28, 4, 4, 128) == (16, 256, False)
-    assert capi.rope_rms_launch_shape(16, 40, 8, 8, 128, kv_fp8=True) == (96, 64, False)
+    assert capi.rope_rms_launch_shape(16, 28, 4, 4, 128) == (16, 256, False, False)
+    assert capi.rope_rms_launch_shape(16, 40, 8, 8, 128, kv_fp8=True) == (96, 64, False, False)
     # fp32 activations: a wave per 512/D Q/K heads, and per 512 elements of the V row when a cache is written
-    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32) == (5, 256, True)
-    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32, set_kv=False) == (3, 256, True)
-    assert capi.rope_rms_launch_shape(4, 7, 2, 3, 256, dtype=torch.float64) == (7, 256, True)
+    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32) == (5, 256, True, False)
+    assert capi.rope_rms_launch_shape(10, 4, 2, 2, 64, dtype=torch.float32, set_kv=False) == (3, 256, True, False)
+    assert capi.rope_rms_launch_shape(4, 7, 2, 3, 256, dtype=torch.float64) == (7, 256, True, False)
     import ctypes as C
     L = capi.lib()
-    o = [C.c_int(0) for _ in range(3)]
+    o = [C.c_int(0) for _ in range(4)]
     refs = [C.byref(x) for x in o]
     assert L.gpuk_rope_rms_launch_shape(0, 32, 8, 8, 128, 1, 0, 1, 0, *refs) == 1
     assert L.gpuk_rope_rms_launch_shape(4, 32, 8, 8, 96, 1, 0, 1, 0, *refs) == 2

@@ -294,8 +294,8 @@ def test_one_wave_per_token_kernel(device, case, gate):
         capi.set_tuning("rope_token_waves", 2)
         capi.set_tuning("rope_token_gate", gate)
         n_axes = 1
-        groups, lanes, _ = capi.rope_rms_launch_shape(tokens, *heads, 128, n_axes, inp.qkv.dtype, True, fp8)
-        assert (groups, lanes) == ((tokens + 3) // 4, 256), "the case must reach the kernel under test"
+        groups, lanes, _, token_waves = capi.rope_rms_launch_shape(tokens, *heads, 128, n_axes, inp.qkv.dtype, True, fp8)
+        assert token_waves and (groups, lanes) == ((tokens + 3) // 4, 256), "the case must reach the kernel under test"
         got = run_set_kv(inp, device)
     finally:
         capi.set_tuning("rope_token_waves", 0)
@@ -306,14 +306,35 @@ def test_one_wave_per_token_kernel(device, case, gate):
     check_set_kv(inp, got, f"[token waves {case}]")
 
 
+@pytest.mark.parametrize("gate", [0, 1, 400])
+def test_unit_kernel_store_gate_changes_no_bits(device, gate):
+    """The kernel with one wave per group of heads holds its stores back, where all of its waves are resident at
+    once (one position axis, a cache write), until the launch's reads are through.  Forced onto small batches: no
+    gate, the shortest, 4 us -- the oracle's bits every time; with three position axes or in place the key is
+    ignored and the bits are the oracle's too."""
+    from gpuk_amd import capi
+
+    print(f"case unit kernel gate {gate}", flush=True)
+    capi.set_tuning("rope_unit_gate", gate)
+    capi.set_tuning("rope_token_waves", 1)
+    try:
+        for heads, mrope, fp8 in (((32, 8, 8), False, False), ((64, 8, 8), False, True), ((28, 4, 4), True, False)):
+            inp = make(77, heads[0], 128, True, seed=31 + gate, mrope=mrope, fp8=fp8, hk=heads[1], hv=heads[2])
+            check_set_kv(inp, run_set_kv(inp, device), f"[unit gate {gate} {heads}]")
+            check_inplace(inp, run_inplace(inp, device), f"[unit gate {gate} {heads} in place]")
+    finally:
+        capi.set_tuning("rope_unit_gate", -1)
+        capi.set_tuning("rope_token_waves", 0)
+
+
 def test_one_wave_per_token_kernel_by_rule(device):
     """The launcher's rule takes that kernel where its waves fill the SIMDs evenly, three or four on each (2900 and
     4000 tokens here), and not in between (3500) or with an fp8 cache; every choice meets the oracle."""
     from gpuk_amd import capi
 
     for tokens, fp8, expect in ((2900, False, True), (3500, False, False), (4000, False, True), (4000, True, False)):
-        groups, lanes, _ = capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 1, torch.bfloat16, True, fp8)
-        assert ((groups, lanes) == ((tokens + 3) // 4, 256)) == expect, (tokens, fp8, groups, lanes)
+        groups, lanes, _, token_waves = capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 1, torch.bfloat16, True, fp8)
+        assert token_waves == expect and (not expect or (groups, lanes) == ((tokens + 3) // 4, 256)), (tokens, fp8, groups, lanes)
         inp = make(tokens, 28, 128, True, seed=tokens + 1, fp8=fp8, hk=4, hv=4)
         check_set_kv(inp, run_set_kv(inp, device), f"[rule T={tokens} fp8={fp8}]")
 
