@@ -92,7 +92,7 @@ struct MaxOp {  // used on magnitudes only, so 0 is the identity.  Compared as b
                 // these order like the values, and a (positive) NaN beats everything, as in the reference's amax
     static __device__ __forceinline__ float apply(float a, float b) {
         const uint32_t x = __builtin_bit_cast(uint32_t, a), y = __builtin_bit_cast(uint32_t, b);
-        return __builtin_bit_cast(float, x > y ? x : y);
+        return __builtin_bit_cast(float, __builtin_elementwise_max(x, y));
     }
     static __device__ __forceinline__ float identity() { return 0.f; }
 };

@@ -218,10 +218,16 @@ int gpuk_increment_floats(float *data, int64_t n, void *stream);
 /* Launch-shape knobs for sweeps and for the tests that show the results do not depend on them; value 0 restores
  * the built-in choice.  Keys: "norm_quant_nchunk" (1/2/4/8 16-byte chunks per lane), "norm_quant_threads" (lanes
  * per row), "norm_quant_row_group_shift" (log2 of the run of consecutive rows one XCD takes; -1, not 0, restores the
- * built-in rule), "rope_block_threads" (64/128/256/512 lanes per workgroup of the rope kernel), "rope_stream_rows" (output rows of
+ * built-in rule), "norm_quant_gate" (how long, in ticks of 10 ns after a wave's entry, the stores of the norm-quant
+ * kernel are held back so that the reads of a batch the chip holds at once go first: -1 the built-in rule, 0 never),
+ * "rope_block_threads" (64/128/256/512 lanes per workgroup of the rope kernel), "rope_stream_rows" (output rows of
  * the rope kernels stored past the L2: 1 never, 2 always), "rope_merge_rows" (1: never let the lanes of an mRoPE
- * token load their cos/sin pieces straight from the row of their axis).  Unknown keys or values return GPUK_ERR_INVALID_ARG.  The settings are process-global plain variables
- * read at launch: set them from one thread while no other thread is launching.  Not part of the reference. */
+ * token load their cos/sin pieces straight from the row of their axis), "rope_token_waves" (the kernel in which one
+ * wave takes a whole token: 1 never, 2 wherever the shape fits it), "rope_token_gate" and "rope_unit_gate" (the
+ * store gate of the two rope kernels, in ticks as above: -1 the built-in rule, 0 never).  The results do not depend
+ * on any of them.  Unknown keys or values return GPUK_ERR_INVALID_ARG.  The settings are process-global plain
+ * variables read at launch: set them from one thread while no other thread is launching.  Not part of the
+ * reference. */
 int gpuk_set_tuning(const char *key, int value);
 
 #ifdef __cplusplus
