@@ -58,6 +58,17 @@ struct RopeArgs {
     uint32_t gate;         // ticks of 10 ns after a wave's entry before which it stores nothing (0 = no gate)
 };
 
+// A pointer read from the argument block by hand is a generic one to the compiler; these say what it points at, so
+// that the accesses through it are global (not flat) ones, and scalar ones where the address is the same in every lane.
+template <typename P>
+__device__ __forceinline__ P *as_global(P *p) {
+    return (P *)(__attribute__((address_space(1))) P *)p;
+}
+template <typename P>
+__device__ __forceinline__ P load_unchanging(const P *p) {  // memory no kernel of the launch writes
+    return *(const __attribute__((address_space(4))) P *)p;
+}
+
 // dword mask selecting the 16-bit halves whose bit is set in a 2-bit field
 __device__ __forceinline__ uint32_t halves_mask(uint32_t two_bits) {
     return ((two_bits & 1u) ? 0x0000ffffu : 0u) | ((two_bits & 2u) ? 0xffff0000u : 0u);
@@ -203,7 +214,7 @@ __device__ __forceinline__ void store_pair(void *p, const u32x4 &a, const u32x4 
 struct UnitState {
     uint32_t t, u;
     int head;
-    bool live, active, is_q;
+    bool active, is_q;
     int64_t slot, p0, p1, p2;
     const uint16_t *token_in;
     u32x4 xa, xb, wa, wb, cosv, sinv, vchunk;
@@ -221,18 +232,9 @@ struct RopeUnit {
     static __device__ __forceinline__ int c0(int sub) { return 8 * sub; }
     static __device__ __forceinline__ int c1(int sub) { return HALF + 8 * sub; }
 
-    // Issues every load of the unit; nothing is waited for.
-    static __device__ __forceinline__ void issue_loads(const RopeArgs &a, uint32_t unit, int lane, UnitState &st) {
-        st.live = unit < a.total_units;  // wave-uniform
-        if (!st.live) return;
-        // With three position axes both weight pointers are pinned in scalar registers, here, ahead of every other
-        // load: the select between the two kernel arguments is otherwise turned into a per-lane load of the pointer
-        // from the argument segment in those instantiations, and the weights wait for that round trip (30.0 -> 27.0
-        // us at 8192 tokens of 28+4 heads, together with the bitmap words of trig_bits).  The one-axis instantiations
-        // keep the pointers in scalar registers by themselves and lose 2-7 % to the pin.  (Not volatile: a volatile
-        // statement ahead of them turns the position loads into vector loads.)
-        const void *qw = a.qw, *kw = a.kw;
-        if constexpr (AXES == 3) asm("" : "+s"(qw), "+s"(kw));
+    // Issues the loads of the unit that need nothing but the kernel's leading parameters (which a wave finds in its
+    // registers): the activations, the unit's share of the V row, the position(s).  Nothing is waited for.
+    static __device__ __forceinline__ void issue_early_loads(const RopeArgs &a, uint32_t unit, int lane, UnitState &st) {
         st.t = a.upt_magic ? __umulhi(unit, a.upt_magic) : unit;
         st.u = unit - st.t * a.units_per_token;
         const int sub = lane % LPH, hl = lane / LPH;
@@ -256,22 +258,32 @@ struct RopeUnit {
             if (v_first < a.hv * (D / 8))
                 st.vchunk = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(st.token_in + (int64_t)heads_qk * D + 8 * v_first));
         }
-        st.p0 = a.positions[(int64_t)st.t * a.ps_token];
+        // (read as memory that no kernel of the launch writes: scalar loads whatever else the kernel contains)
+        st.p0 = load_unchanging(a.positions + (int64_t)st.t * a.ps_token);
         if constexpr (AXES == 3) {
-            st.p1 = a.positions[a.ps_axis + (int64_t)st.t * a.ps_token];
-            st.p2 = a.positions[2 * a.ps_axis + (int64_t)st.t * a.ps_token];
+            st.p1 = load_unchanging(a.positions + a.ps_axis + (int64_t)st.t * a.ps_token);
+            st.p2 = load_unchanging(a.positions + 2 * a.ps_axis + (int64_t)st.t * a.ps_token);
         }
-        // so far nothing needed more than the kernel's leading parameters, which a wave finds in its registers; the
-        // slot and the weights are reached through pointers of the argument block
-        if constexpr (SETKV) st.slot = a.kv_loc[st.t];
+    }
+
+    // The loads reached through pointers of the argument block: the token's cache slot and the norm weights.
+    static __device__ __forceinline__ void issue_late_loads(const RopeArgs &a, int lane, UnitState &st) {
+        // With three position axes both weight pointers are pinned in scalar registers: the select between the two
+        // kernel arguments is otherwise turned into a per-lane load of the pointer from the argument segment in those
+        // instantiations, and the weights wait for that round trip.  The one-axis instantiations keep the pointers in
+        // scalar registers by themselves and lose 2-7 % to the pin.
+        const void *qw = a.qw, *kw = a.kw;
+        if constexpr (AXES == 3) asm("" : "+s"(qw), "+s"(kw));
+        const int sub = lane % LPH;
+        if constexpr (SETKV) st.slot = load_unchanging(a.kv_loc + st.t);
+        typedef const __attribute__((address_space(1))) u32x4 *GlobalChunk;
         const uint16_t *wsrc = static_cast<const uint16_t *>(st.is_q ? qw : kw);
-        st.wa = *reinterpret_cast<const u32x4 *>(wsrc + c0(sub));
-        st.wb = *reinterpret_cast<const u32x4 *>(wsrc + c1(sub));
+        st.wa = *(GlobalChunk)(wsrc + c0(sub));
+        st.wb = *(GlobalChunk)(wsrc + c1(sub));
     }
 
     // The cos/sin loads, whose addresses wait for the positions.
     static __device__ __forceinline__ void issue_table_loads(const RopeArgs &a, int lane, UnitState &st) {
-        if (!st.live) return;
         const int sub = lane % LPH;
         const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin);
         const int64_t p0 = st.p0;
@@ -321,7 +333,6 @@ struct RopeUnit {
     // time (a template parameter: as a run-time choice the check cost the launches without a gate 2-6 %).
     template <bool GATED>
     static __device__ __forceinline__ void finish(const RopeArgs &a, int lane, UnitState &st, uint64_t entry) {
-        if (!st.live) return;
         const int sub = lane % LPH;
         const int heads_qk = a.hq + a.hk, heads_all = heads_qk + a.hv;
         const u32x4 &xa = st.xa, &xb = st.xb, &wa = st.wa, &wb = st.wb, &cosv = st.cosv, &sinv = st.sinv;
@@ -387,6 +398,17 @@ struct RopeUnit {
 // (The three-axis instantiations take 66 registers per lane, one wave short of the eight a SIMD can hold; held to 64
 // with amdgpu_waves_per_eu they fit without spilling and run 1-4 % slower: 26.9 against 26.6 us at 8192 tokens of
 // 28+4+4 heads, 51.3 against 49.1 at 16384.)
+// The leading parameters of the kernel below as the argument segment lays them out; the block follows them.
+struct UnitKernelLead {
+    const void *qkv_in;
+    const int64_t *positions;
+    uint32_t total_units, units_per_token, upt_magic;
+    int hq, hk;
+    uint32_t hv_and_waves;
+    int64_t ps_token, ps_axis;
+};
+static_assert(sizeof(UnitKernelLead) == 56 && sizeof(UnitKernelLead) % alignof(RopeArgs) == 0, "offset of the block");
+
 template <typename T, int D, bool NEOX, int AXES, bool SETKV, bool KVFP8, bool GATED>
 __global__ void __launch_bounds__(512)
 rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_units, uint32_t units_per_token,
@@ -397,7 +419,7 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
     const uint32_t unit = (blockIdx.x << (hv_and_waves >> 24)) + wave;
     if (unit >= total_units) return;
     const uint64_t entry = GATED ? __builtin_amdgcn_s_memrealtime() : 0;
-    RopeArgs a = rest;  // the fields that came ahead replace their copies in the block
+    RopeArgs a;
     a.qkv_in = qkv_in;
     a.positions = positions;
     a.total_units = total_units;
@@ -411,9 +433,45 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
     GPUK_STAMPS_BEGIN();  // profiling build only
     const int lane = threadIdx.x & 63;
     UnitState st;
-    Unit::issue_loads(a, unit, lane, st);
+    Unit::issue_early_loads(a, unit, lane, st);
+    // The rest of the arguments is fetched from the argument block only now, behind the requests above.  (Left to
+    // the compiler the fetch is the kernel's first instruction, and the first vector load then waits for it: in one
+    // instantiation for a register the fetch is about to overwrite, in another for the pinned weight pointers.)
+    // (`rest` is read through the argument segment's own address: taking the parameter's address would have the
+    // whole block copied to the stack.  It follows the 14 leading dwords.)
+    typedef const __attribute__((address_space(4))) RopeArgs *BlockPtr;
+    BlockPtr block = (BlockPtr)((const __attribute__((address_space(4))) char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                sizeof(UnitKernelLead));
+    asm volatile("" : "+s"(block));
+    a.kv_loc = as_global(block->kv_loc);
+    a.qkv_out = as_global(block->qkv_out);
+    a.qw = as_global(block->qw);
+    a.kw = as_global(block->kw);
+    a.cos_sin = as_global(block->cos_sin);
+    a.q_out = as_global(block->q_out);
+    a.k_cache = as_global(block->k_cache);
+    a.v_cache = as_global(block->v_cache);
+    a.eps = block->eps;
+    a.k_scale = block->k_scale;
+    a.v_scale = block->v_scale;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a.axis1[i] = block->axis1[i];
+        a.axis2[i] = block->axis2[i];
+    }
+    a.stream_rows = block->stream_rows;
+    a.merge_rows = block->merge_rows;
+    a.gate = block->gate;
+    // ... all of it in one go (the compiler otherwise fetches each field where it is first used, the output pointers
+    // after the arithmetic, and the wave waits for the scalar cache once more before it can store)
+    asm volatile("" ::"s"(a.kv_loc), "s"(a.qkv_out), "s"(a.qw), "s"(a.kw), "s"(a.cos_sin), "s"(a.q_out), "s"(a.k_cache),
+                 "s"(a.v_cache), "s"(a.eps), "s"(a.k_scale), "s"(a.v_scale), "s"(a.stream_rows), "s"(a.merge_rows),
+                 "s"(a.gate));
+    Unit::issue_late_loads(a, lane, st);
     GPUK_STAMP(1);  // activations, weights, position and slot requested
     Unit::issue_table_loads(a, lane, st);
+    // (the slot is asked for here and not where the rows are stored, for the same reason)
+    if constexpr (SETKV) asm volatile("" ::"s"((uint32_t)st.slot), "s"((uint32_t)(st.slot >> 32)));
     GPUK_STAMP(2);  // position known, cos/sin requested
     // Every load of the wave is in flight before the first use of any of them: without this fence the scheduler
     // moves arithmetic above later loads and the wave pays several memory round trips in a row.
@@ -440,6 +498,16 @@ constexpr uint32_t kTokenWaveCapacity = 4096;  // 4 waves per SIMD: the 100-odd 
 // (measured at 2900-4096 tokens of 28+4+4 and 32+8+8 heads: 3-7 % ahead of the kernel above with this gate, 2-4 %
 // with the full time, level or behind with 0.8 or 1.1 times it, and 6 % behind it with no gate at all).
 constexpr double kGateBytesPerTick = 70000.0 / 0.9;
+
+// The leading parameters of the kernel below as the argument segment lays them out; the block follows them.
+struct TokenKernelLead {
+    const void *qkv_in;
+    const int64_t *positions;
+    uint32_t num_tokens, gate;
+    int hq, hk, hv;
+    int64_t ps_token;
+};
+static_assert(sizeof(TokenKernelLead) == 48 && sizeof(TokenKernelLead) % alignof(RopeArgs) == 0, "offset of the block");
 
 template <typename T, int D, bool NEOX, int UPT, bool KVFP8>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
@@ -468,17 +536,36 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
         const int c = min(lane + 64 * j, v_chunks - 1);  // the host admits at most 128 chunks of V per token
         v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(token_in + (int64_t)heads_qk * D + 8 * c));
     }
-    const int64_t p0 = positions[(int64_t)t * ps_token];
-    const int64_t slot = rest.kv_loc[t];
-    const uint16_t *qw = static_cast<const uint16_t *>(rest.qw), *kw = static_cast<const uint16_t *>(rest.kw);
+    const int64_t p0 = load_unchanging(positions + (int64_t)t * ps_token);
+    // the rest of the arguments, fetched from the argument block behind the requests above (see rope_rms_kernel)
+    typedef const __attribute__((address_space(4))) RopeArgs *BlockPtr;
+    BlockPtr block = (BlockPtr)((const __attribute__((address_space(4))) char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                sizeof(TokenKernelLead));
+    asm volatile("" : "+s"(block));
+    RopeArgs a;
+    a.kv_loc = as_global(block->kv_loc);
+    a.qw = as_global(block->qw);
+    a.kw = as_global(block->kw);
+    a.cos_sin = as_global(block->cos_sin);
+    a.q_out = as_global(block->q_out);
+    a.k_cache = as_global(block->k_cache);
+    a.v_cache = as_global(block->v_cache);
+    a.eps = block->eps;
+    a.k_scale = block->k_scale;
+    a.v_scale = block->v_scale;
+    asm volatile("" ::"s"(a.kv_loc), "s"(a.qw), "s"(a.kw), "s"(a.cos_sin), "s"(a.q_out), "s"(a.k_cache), "s"(a.v_cache),
+                 "s"(a.eps), "s"(a.k_scale), "s"(a.v_scale));
+    const int64_t slot = load_unchanging(a.kv_loc + t);
+    const uint16_t *qw = static_cast<const uint16_t *>(a.qw), *kw = static_cast<const uint16_t *>(a.kw);
     const u32x4 qwa = *reinterpret_cast<const u32x4 *>(qw + 8 * sub), qwb = *reinterpret_cast<const u32x4 *>(qw + HALF + 8 * sub);
     const u32x4 kwa = *reinterpret_cast<const u32x4 *>(kw + 8 * sub), kwb = *reinterpret_cast<const u32x4 *>(kw + HALF + 8 * sub);
-    const uint16_t *row = static_cast<const uint16_t *>(rest.cos_sin) + p0 * D;
+    const uint16_t *row = static_cast<const uint16_t *>(a.cos_sin) + p0 * D;
     const u32x4 cosv = load_trig<D, NEOX>(row, sub), sinv = load_trig<D, NEOX>(row + HALF, sub);
+    asm volatile("" ::"s"((uint32_t)slot), "s"((uint32_t)(slot >> 32)));  // asked for here, not where the rows are stored
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- norm and rotation, unit by unit, in place
-    const float eps = rest.eps;
+    const float eps = a.eps;
 #pragma unroll
     for (int u = 0; u < UPT; ++u) {
         const int h0 = u * HPW;
@@ -504,13 +591,13 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
     for (int u = 0; u < UPT; ++u) {
         const int head = u * HPW + hl;
         if (head < hq) {
-            uint16_t *dst = static_cast<uint16_t *>(rest.q_out) + ((int64_t)t * hq + head) * D + 8 * sub;
+            uint16_t *dst = static_cast<uint16_t *>(a.q_out) + ((int64_t)t * hq + head) * D + 8 * sub;
             store_pair<HALF * 2>(dst, xa[u], xb[u], true);
         } else if (head < heads_qk && slot_ok) {
             const int64_t at = (slot * hk + (head - hq)) * D + 8 * sub;
             if constexpr (KVFP8) {
-                uint8_t *dst = static_cast<uint8_t *>(rest.k_cache) + at;
-                const float s = rest.k_scale, rcp = 1.0f / s;
+                uint8_t *dst = static_cast<uint8_t *>(a.k_cache) + at;
+                const float s = a.k_scale, rcp = 1.0f / s;
                 if (scale_is_fast(s)) {
                     *reinterpret_cast<u32x2 *>(dst) = quantize_chunk<T, true>(xa[u], s, rcp);
                     *reinterpret_cast<u32x2 *>(dst + HALF) = quantize_chunk<T, true>(xb[u], s, rcp);
@@ -519,7 +606,7 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
                     *reinterpret_cast<u32x2 *>(dst + HALF) = quantize_chunk<T, false>(xb[u], s, rcp);
                 }
             } else {
-                store_pair<HALF * 2>(static_cast<uint16_t *>(rest.k_cache) + at, xa[u], xb[u], true);
+                store_pair<HALF * 2>(static_cast<uint16_t *>(a.k_cache) + at, xa[u], xb[u], true);
             }
         }
     }
@@ -529,11 +616,11 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
         if (slot_ok && c < v_chunks) {
             const int64_t off = slot * hv * D + 8 * (int64_t)c;
             if constexpr (KVFP8) {
-                const float s = rest.v_scale, rcp = 1.0f / s;
-                *reinterpret_cast<u32x2 *>(static_cast<uint8_t *>(rest.v_cache) + off) =
+                const float s = a.v_scale, rcp = 1.0f / s;
+                *reinterpret_cast<u32x2 *>(static_cast<uint8_t *>(a.v_cache) + off) =
                     scale_is_fast(s) ? quantize_chunk<T, true>(v[j], s, rcp) : quantize_chunk<T, false>(v[j], s, rcp);
             } else {
-                *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(rest.v_cache) + off) = v[j];
+                *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(a.v_cache) + off) = v[j];
             }
         }
     }
