@@ -938,7 +938,7 @@ int g_merge_rows = 0;     // mRoPE rows merged on load where the sections allow:
 int g_token_waves = 0;    // one-wave-per-token kernel: 0 = built-in rule, 1 = never, 2 = wherever it fits
 int g_token_gate = -1;    // its gate in ticks of 10 ns; -1 = from the bytes of the call
 int g_unit_gate = -1;     // gate of the kernel with one wave per unit: -1 = built-in rule, 0 = none, > 0 = ticks
-constexpr uint32_t kTokenWaveMinTokens = 2800;
+constexpr uint32_t kResidentUnits = 8192;  // waves of the one-wave-per-unit kernel the chip holds at once (8 per SIMD)
 
 // Streaming stores, measured on MI355X (32/8/8, 28/4/4 and 64/8/8 heads, head sizes 64-256, random slots): q_out /
 // K rows / in-place rows written past the L2 are ahead from about 10 MB per call on (64+8 heads, fp8 cache: 5.9
@@ -962,23 +962,28 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     const int64_t read_bytes = 2 * (int64_t)a.num_tokens * (a.hq + a.hk + a.hv) * D;
     const bool fits = axes == 1 && set_kv && D == 128 && a.units_per_token >= 4 && a.units_per_token <= 5 &&
                       a.hv * (D / 8) <= 128 && a.hv > 0 && a.num_tokens <= kTokenWaveCapacity;
-    // ... and where its waves fill the SIMDs evenly, three or four on each: with a SIMD in four holding a wave fewer
-    // the launch waits for the fuller ones (3700 tokens: 1-3 % behind the kernel above; 1024-2048 tokens: level)
-    const uint32_t rounds = (a.num_tokens + 1023) / 1024;
-    const bool even = a.num_tokens >= kTokenWaveMinTokens && 100 * (uint64_t)a.num_tokens >= 94 * (uint64_t)rounds * 1024;
-    p.token_waves = fits && (g_token_waves == 2 || (g_token_waves == 0 && even && !kv_fp8));
+    // ... and too large for the kernel above to hold all of its waves at once (more than 8192 units; below that the
+    // kernel above, gated, is ahead: 8.3 against 9.7 us at 1536 tokens of 32+8+8 heads; from there on this one is,
+    // 9.9 against 10.1 us at 1800 tokens, 10.3 against 11.1 at 2048, 13.6 against 14.8 at 3000, 16.6 against 17.3 at
+    // 3700, 17.4 against 18.8 at 4096; 28+4+4 heads: 11.0 against 11.9 us at 3000 tokens).  Not with an fp8 cache,
+    // whose conversions lengthen the wave (32+8+8 heads: 15.7 against 14.4 us at 3000 tokens, 19.9 against 18.3 at 4096).
+    const bool large = a.total_units > kResidentUnits;
+    p.token_waves = fits && (g_token_waves == 2 || (g_token_waves == 0 && large && !kv_fp8));
     const double gate = g_token_gate >= 0 ? (double)g_token_gate : (double)read_bytes / kGateBytesPerTick;
     p.gate = (uint32_t)std::min(gate, 5000.0);
     // The kernel with one wave per unit gates its stores in the same way where its waves are all resident at once
-    // (8192 of them, eight per SIMD, with one position axis) and fill at least half of that round; the gate is the
-    // read time at 7 TB/s.  Measured with a cache write: 64+8+8 heads, fp8 cache, 7.7 against 8.5 us at 768 tokens, 8.6
-    // against 9.5 at 900; 32+8+8 heads 6.1 against 7.0 us at 1024 tokens, 8.4 against 9.5 at 1600; nothing to gain
-    // below half a round, 15-35 % slower one unit beyond it (10.4 -> 11.9 us at 1024 tokens of 64+8+8 heads), and
-    // 2 % at best with three position axes, whose instantiations hold seven waves per SIMD.
+    // (8192 of them, eight per SIMD, with one position axis) and fill at least half of that round; the gate is 0.85
+    // of the read time at 7 TB/s, 0.7 of it with an fp8 cache (half the bytes to write) and then only from 0.7 of a
+    // round on.  Measured with a cache write: 64+8+8 heads, 16-bit cache, 7.1 against 7.8 us at 768 tokens, 7.8 against
+    // 8.9 at 900; fp8 cache, 7.4 against 7.9 us at 768 tokens, 8.2 against 8.7 at 900, but 5.9 against 5.8 at 512;
+    // 32+8+8 heads, 16-bit cache, 6.4 against 6.7 us at 1024 tokens, 8.3 against 9.1 at 1536; nothing to gain below
+    // half a round, 15-35 % slower one unit beyond a round, and 2 % at best with three position axes, whose
+    // instantiations hold seven waves per SIMD.
     p.unit_gate = 0;
     if (g_unit_gate > 0) p.unit_gate = (uint32_t)g_unit_gate;
-    else if (g_unit_gate < 0 && axes == 1 && set_kv && a.total_units <= 8192 && a.total_units >= 4096)
-        p.unit_gate = (uint32_t)std::min((double)read_bytes / 70000.0, 5000.0);
+    else if (g_unit_gate < 0 && axes == 1 && set_kv && a.total_units <= kResidentUnits &&
+             a.total_units >= (kv_fp8 ? kResidentUnits * 7 / 10 : kResidentUnits / 2))
+        p.unit_gate = (uint32_t)std::min((kv_fp8 ? 0.7 : 0.85) * (double)read_bytes / 70000.0, 5000.0);
     // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
     const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
     const int64_t call_bytes = set_kv ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +

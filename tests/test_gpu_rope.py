@@ -274,8 +274,8 @@ TOKEN_WAVE_CASES = [
 @pytest.mark.parametrize("case", range(len(TOKEN_WAVE_CASES)))
 @pytest.mark.parametrize("gate", [-1, 0, 700])
 def test_one_wave_per_token_kernel(device, case, gate):
-    """Batches that fit the chip in one round (2800-4096 tokens of 25-40 Q and K heads, one position axis, a cache)
-    run a kernel in which a wave takes a whole token, asks for everything it reads at once and holds its stores back
+    """Batches of up to 4096 tokens (25-40 Q and K heads, one position axis, a cache) that the other kernel cannot hold
+    in one round run a kernel in which a wave takes a whole token, asks for everything it reads at once and holds its stores back
     until the launch's reads are through.  Forced onto small batches here, with the gate it would compute, none, and a
     long one (7 us): the oracle's bits, and the same bits as the kernel with one wave per group of heads."""
     from gpuk_amd import capi
@@ -328,11 +328,13 @@ def test_unit_kernel_store_gate_changes_no_bits(device, gate):
 
 
 def test_one_wave_per_token_kernel_by_rule(device):
-    """The launcher's rule takes that kernel where its waves fill the SIMDs evenly, three or four on each (2900 and
-    4000 tokens here), and not in between (3500) or with an fp8 cache; every choice meets the oracle."""
+    """The launcher's rule takes that kernel where the other one could not hold all of its waves at once (more than
+    8192 groups of heads: 2049 tokens of 28+4 heads, not 2048) up to the 4096 tokens it holds itself, and not with an
+    fp8 cache; every choice meets the oracle."""
     from gpuk_amd import capi
 
-    for tokens, fp8, expect in ((2900, False, True), (3500, False, False), (4000, False, True), (4000, True, False)):
+    for tokens, fp8, expect in ((2048, False, False), (2049, False, True), (3500, False, True), (4096, False, True),
+                                (4097, False, False), (4000, True, False)):
         groups, lanes, _, token_waves = capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 1, torch.bfloat16, True, fp8)
         assert token_waves == expect and (not expect or (groups, lanes) == ((tokens + 3) // 4, 256)), (tokens, fp8, groups, lanes)
         inp = make(tokens, 28, 128, True, seed=tokens + 1, fp8=fp8, hk=4, hv=4)
