@@ -378,7 +378,11 @@ def main():
                     else "rope_rms_kernel (one wave per group of heads)")
             return f"{form}, {groups} workgroups x {lanes} lanes, rows stored {'past the L2' if streamed else 'through the L2'}"
 
-        for name, r in (("rope_kv_qwen3_T4096", workloads.config3()), ("mrope_kv_qwen2vl_T8192", workloads.config4())):
+        # (the third line: the second shape's kernel on text-only positions -- three equal rows, every token one table
+        # row of its own -- at a token count of its own, so that a profiler's per-grid rows tell the two apart: its
+        # fetched bytes beside the second line's show what the table rows of image tokens cost, which is nothing)
+        for name, r in (("rope_kv_qwen3_T4096", workloads.config3()), ("mrope_kv_qwen2vl_T8192", workloads.config4()),
+                        ("mrope_kv_text_only_T8184", workloads.config4(8184, text_only=True))):
             nbytes, avg, med, mn, burst, read_bytes = rope_case(r, 4)
             groups, lanes_b, _, _ = capi.rope_rms_launch_shape(r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v,
                                                             r.head_size, 3 if r.mrope_section is not None else 1,

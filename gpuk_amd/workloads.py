@@ -170,10 +170,11 @@ def vl_positions(num_tokens: int, text_run: int = 1024, grid: int = 32) -> torch
     return torch.tensor(rows, dtype=torch.int64).contiguous()
 
 
-def config4(num_tokens: int = 8192, is_interleaved: bool = False) -> RopeInputs:
-    """Qwen2-VL-like mRoPE: Hq=28, Hk=Hv=4, D=128, sections [16,24,24], text + 32x32 image segments."""
+def config4(num_tokens: int = 8192, is_interleaved: bool = False, text_only: bool = False) -> RopeInputs:
+    """Qwen2-VL-like mRoPE: Hq=28, Hk=Hv=4, D=128, sections [16,24,24], text + 32x32 image segments
+    (text_only: one run of text, the three position rows equal)."""
     inp = rope_inputs(num_tokens, 28, 4, 4, 128, seed=4, max_pos=32768, num_slots=max(num_tokens, 16) * 2)
-    inp.positions = vl_positions(num_tokens)
+    inp.positions = vl_positions(num_tokens, text_run=num_tokens if text_only else 1024)
     inp.mrope_section = [16, 24, 24]
     inp.is_interleaved = is_interleaved
     return inp

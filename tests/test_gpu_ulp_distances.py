@@ -88,6 +88,16 @@ def test_rope_distances_from_the_unmoved_oracle(device, case):
     assert (dq == 0).float().mean().item() >= 0.999 and (dk == 0).float().mean().item() >= 0.999
     assert (dq <= 1).float().mean().item() >= 1 - 2e-5 and (dk <= 1).float().mean().item() >= 1 - 2e-5
     assert beyond_q <= max(2 * seen_q, 8) and beyond_k <= max(2 * seen_k, 8), (beyond_q, beyond_k)
+    # ... and every element, however small, lies within 2 ULPs *of its head's largest value* of the unmoved oracle: an
+    # rstd one fp32 ULP away moves a normed value by at most one ULP of itself, the rotation adds two of those
+    qf, rf = q_out.cpu().float().reshape(-1, D), q_ref.float().reshape(-1, D)
+    head_ulp = torch.exp2(torch.floor(torch.log2(rf.abs().amax(dim=1, keepdim=True).clamp_min(1e-30))) - 7)
+    worst_abs = ((qf - rf).abs() / head_ulp).max().item()
+    print(f"[ULP] kernel B {name}, q_out: worst distance in ULPs of the head's largest value {worst_abs:.3f}; "
+          f"worst in ULPs of the element itself {worst_q}", flush=True)
+    assert worst_abs <= 2.0 and worst_q <= 64
     if fp8:
         assert worst_k <= 1
+    else:
+        assert worst_k <= 64
     assert torch.equal(vc.cpu()[loc].view(torch.uint8), v_ref[loc].view(torch.uint8))
