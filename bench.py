@@ -374,8 +374,9 @@ def main():
             groups, lanes, streamed, token_waves = capi.rope_rms_launch_shape(
                 r.num_tokens, r.num_heads_q, r.num_heads_k, r.num_heads_v, r.head_size,
                 3 if r.mrope_section is not None else 1, torch.bfloat16, True, r.kv_dtype == torch.float8_e4m3fn)
-            form = ("rope_rms_token_kernel (one wave per token, stores gated behind the launch's reads)" if token_waves
-                    else "rope_rms_kernel (one wave per group of heads)")
+            form = ("rope_rms_kernel (one wave per group of heads)", "rope_rms_token_kernel (one wave per token, stores gated "
+                    "behind the launch's reads)", "rope_rms_token_kernel (one wave per two tokens, the second through LDS; "
+                    "stores gated behind the launch's reads)")[token_waves]
             return f"{form}, {groups} workgroups x {lanes} lanes, rows stored {'past the L2' if streamed else 'through the L2'}"
 
         # (the third line: the second shape's kernel on text-only positions -- three equal rows, every token one table

@@ -126,13 +126,14 @@ def add_rmsnorm_quant_launch_shape(tokens: int, hidden: int, dtype=torch.bfloat1
 
 def rope_rms_launch_shape(num_tokens: int, num_heads_q: int, num_heads_k: int, num_heads_v: int, head_size: int,
                           n_axes: int = 1, dtype=torch.bfloat16, set_kv: bool = True, kv_fp8: bool = False):
-    """(workgroups, lanes per workgroup, streamed, one wave per token) of the launch the rope entry points make."""
+    """(workgroups, lanes per workgroup, streamed, tokens per wave) of the launch the rope entry points make; tokens
+    per wave is 0 for the kernel in which a wave takes a group of heads, 1 or 2 for the one in which it takes tokens."""
     out = [C.c_int(0) for _ in range(4)]
     rc = lib().gpuk_rope_rms_launch_shape(num_tokens, num_heads_q, num_heads_k, num_heads_v, head_size, n_axes,
                                           DTYPE[dtype], int(set_kv), 1 if kv_fp8 else 0, *(C.byref(o) for o in out))
     if rc:
         raise GpukError(rc, "gpuk_rope_rms_launch_shape")
-    return out[0].value, out[1].value, bool(out[2].value), bool(out[3].value)
+    return out[0].value, out[1].value, bool(out[2].value), out[3].value
 
 
 def _pos_args(positions):

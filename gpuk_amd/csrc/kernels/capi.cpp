@@ -46,7 +46,7 @@ extern "C" int gpuk_set_tuning(const char *key, int value) {
         return GPUK_OK;
     }
     if (strcmp(key, "rope_token_waves") == 0) {
-        if (value < 0 || value > 2) return GPUK_ERR_INVALID_ARG;
+        if (value < 0 || value > 3) return GPUK_ERR_INVALID_ARG;
         gpuk::set_rope_tuning(1, value);
         return GPUK_OK;
     }

@@ -484,15 +484,19 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// One wave per token, for batches that the chip holds in one round (one position axis, a cache write, up to
-// kTokenWaveCapacity tokens of UPT units each).  The memory system serves reads and writes one direction at a time,
-// and a kernel of this size (tens of MB each way, 15-20 us) spends a fifth of its time paying for the mix; here the
-// launch is arranged so that there is hardly any: every wave is resident from the start and asks for everything it
-// will read -- all UPT units of its token, its share of nothing but its own token's V row, the weights, then the
-// table row -- before it computes anything, the rotated rows replace the activations in the wave's registers, and
-// no store is issued before `gate` ticks (10 ns) after the wave's entry, the time the launch's reads take at the
-// read-only rate (the host computes it from the bytes of the call).  The chip thus reads for the first half of the
-// launch and writes for the second.  The arithmetic is norm_rotate's, as in the kernel above.
+// One wave per token -- or per two tokens --, for batches that the chip holds in one round (a cache write, up to
+// kTokenWaveCapacity waves).  The memory system serves reads and writes one direction at a time, and a kernel of this
+// size (tens of MB each way, 15-25 us) spends a fifth of its time paying for the mix; here the launch is arranged so
+// that there is hardly any: every wave is resident from the start and asks for everything it will read -- all UPT
+// units of its token, its token's V row, the weights, then the table row -- before it computes anything, the
+// rotated rows replace the activations in the wave's registers, and no store is issued before `gate` ticks (10 ns)
+// after the wave's entry, the time the launch's reads take at the read-only rate (the host computes it from the
+// bytes of the call).  The chip thus reads for the first half of the launch and writes for the second.
+// TWO: the wave takes a second token (the one num_waves further on), whose activations and V row travel from global
+// memory straight into the wave's 9 KB of LDS (global_load_lds_dwordx4: no register is the destination) during the
+// same read phase, and are taken into the first token's registers once that one is stored.  Registers and LDS
+// together hold 8192 tokens of up to 32 Q and K heads and 4 V heads: twice the batch, still one round.
+// The arithmetic is norm_rotate's, as in the kernel above.
 constexpr uint32_t kTokenWaveCapacity = 4096;  // 4 waves per SIMD: the 100-odd registers a wave of this kernel takes
 // The gate: nine tenths of the time the launch's reads take at 7 TB/s, the rate of a read-only kernel on this part
 // (measured at 2900-4096 tokens of 28+4+4 and 32+8+8 heads: 3-7 % ahead of the kernel above with this gate, 2-4 %
@@ -505,67 +509,56 @@ struct TokenKernelLead {
     const int64_t *positions;
     uint32_t num_tokens, gate;
     int hq, hk, hv;
-    int64_t ps_token;
+    uint32_t num_waves;
+    int64_t ps_token, ps_axis;
 };
-static_assert(sizeof(TokenKernelLead) == 48 && sizeof(TokenKernelLead) % alignof(RopeArgs) == 0, "offset of the block");
+static_assert(sizeof(TokenKernelLead) == 56 && sizeof(TokenKernelLead) % alignof(RopeArgs) == 0, "offset of the block");
 
-template <typename T, int D, bool NEOX, int UPT, bool KVFP8>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
-rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num_tokens, uint32_t gate, int hq, int hk,
-                      int hv, int64_t ps_token, const RopeArgs rest) {
-    constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
-    const uint64_t entry = __builtin_amdgcn_s_memrealtime();
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t t = blockIdx.x * 4 + wave;
-    if (t >= num_tokens) return;
-    const int lane = threadIdx.x & 63, sub = lane % LPH, hl = lane / LPH;
-    const int heads_qk = hq + hk, heads_all = heads_qk + hv, v_chunks = hv * (D / 8);
-    const uint16_t *token_in = static_cast<const uint16_t *>(qkv_in) + (int64_t)t * heads_all * D;
+// One 16-byte piece per lane from global memory into LDS at lds_byte_offset + 16 * lane; the address is the lane's
+// own.  M0 carries the LDS offset: one wait state after writing it, and it is named as clobbered so that the compiler
+// never keeps a value of its own there across the transfer (its warning that M0 is reserved is silenced: reserved
+// means it allocates nothing there, which is the point).  Counted by vmcnt like a load.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void lds_fill16(uint32_t lds_byte_offset, const void *lane_address) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 1\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds_byte_offset), "v"(lane_address) : "memory", "m0");
+}
+#pragma clang diagnostic pop
 
-    // ---- everything the wave reads, asked for at once (what needs only the leading parameters first)
-    u32x4 xa[UPT], xb[UPT], v[2];
-#pragma unroll
-    for (int u = 0; u < UPT; ++u) {
-        const int head = min(u * HPW + hl, heads_qk - 1);  // lanes past the last head re-read it
-        const uint16_t *src = token_in + (int64_t)head * D;
-        xa[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 8 * sub));
-        xb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + HALF + 8 * sub));
+// cos and sin pieces of a lane for a token at positions (p0, p1, p2): with three axes every aligned group of 8
+// frequencies takes one axis (the host checks the sections), so each lane reads its pieces from that axis's row
+template <int D, bool NEOX, int AXES>
+__device__ __forceinline__ void load_trig_by_axis(const uint16_t *table, int64_t p0, int64_t p1, int64_t p2,
+                                                  const uint32_t (&axis1)[4], const uint32_t (&axis2)[4], int sub,
+                                                  u32x4 &cosv, u32x4 &sinv) {
+    constexpr int HALF = D / 2;
+    if constexpr (AXES == 1) {
+        cosv = load_trig<D, NEOX>(table + p0 * D, sub);
+        sinv = load_trig<D, NEOX>(table + p0 * D + HALF, sub);
+    } else {
+        const uint32_t b1 = trig_bits<D, NEOX>(axis1, sub), b2 = trig_bits<D, NEOX>(axis2, sub);
+        const int64_t pa = (b2 & 1u) ? p2 : ((b1 & 1u) ? p1 : p0);
+        if constexpr (NEOX) {
+            cosv = load_trig<D, NEOX>(table + pa * D, sub);
+            sinv = load_trig<D, NEOX>(table + pa * D + HALF, sub);
+        } else {
+            const int64_t pb = (b2 & 16u) ? p2 : ((b1 & 16u) ? p1 : p0);
+            const u32x2 cl = *reinterpret_cast<const u32x2 *>(table + pa * D + 4 * sub);
+            const u32x2 ch = *reinterpret_cast<const u32x2 *>(table + pb * D + D / 4 + 4 * sub);
+            const u32x2 sl = *reinterpret_cast<const u32x2 *>(table + pa * D + HALF + 4 * sub);
+            const u32x2 sh = *reinterpret_cast<const u32x2 *>(table + pb * D + HALF + D / 4 + 4 * sub);
+            cosv = u32x4{cl[0], cl[1], ch[0], ch[1]};
+            sinv = u32x4{sl[0], sl[1], sh[0], sh[1]};
+        }
     }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int c = min(lane + 64 * j, v_chunks - 1);  // the host admits at most 128 chunks of V per token
-        v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(token_in + (int64_t)heads_qk * D + 8 * c));
-    }
-    const int64_t p0 = load_unchanging(positions + (int64_t)t * ps_token);
-    // the rest of the arguments, fetched from the argument block behind the requests above (see rope_rms_kernel)
-    typedef const __attribute__((address_space(4))) RopeArgs *BlockPtr;
-    BlockPtr block = (BlockPtr)((const __attribute__((address_space(4))) char *)__builtin_amdgcn_kernarg_segment_ptr() +
-                                sizeof(TokenKernelLead));
-    asm volatile("" : "+s"(block));
-    RopeArgs a;
-    a.kv_loc = as_global(block->kv_loc);
-    a.qw = as_global(block->qw);
-    a.kw = as_global(block->kw);
-    a.cos_sin = as_global(block->cos_sin);
-    a.q_out = as_global(block->q_out);
-    a.k_cache = as_global(block->k_cache);
-    a.v_cache = as_global(block->v_cache);
-    a.eps = block->eps;
-    a.k_scale = block->k_scale;
-    a.v_scale = block->v_scale;
-    asm volatile("" ::"s"(a.kv_loc), "s"(a.qw), "s"(a.kw), "s"(a.cos_sin), "s"(a.q_out), "s"(a.k_cache), "s"(a.v_cache),
-                 "s"(a.eps), "s"(a.k_scale), "s"(a.v_scale));
-    const int64_t slot = load_unchanging(a.kv_loc + t);
-    const uint16_t *qw = static_cast<const uint16_t *>(a.qw), *kw = static_cast<const uint16_t *>(a.kw);
-    const u32x4 qwa = *reinterpret_cast<const u32x4 *>(qw + 8 * sub), qwb = *reinterpret_cast<const u32x4 *>(qw + HALF + 8 * sub);
-    const u32x4 kwa = *reinterpret_cast<const u32x4 *>(kw + 8 * sub), kwb = *reinterpret_cast<const u32x4 *>(kw + HALF + 8 * sub);
-    const uint16_t *row = static_cast<const uint16_t *>(a.cos_sin) + p0 * D;
-    const u32x4 cosv = load_trig<D, NEOX>(row, sub), sinv = load_trig<D, NEOX>(row + HALF, sub);
-    asm volatile("" ::"s"((uint32_t)slot), "s"((uint32_t)(slot >> 32)));  // asked for here, not where the rows are stored
-    __builtin_amdgcn_sched_barrier(0);
+}
 
-    // ---- norm and rotation, unit by unit, in place
-    const float eps = a.eps;
+// Norm and rotation of a token's units, in place.
+template <typename T, int D, bool NEOX, int UPT>
+__device__ __forceinline__ void token_rotate(u32x4 (&xa)[UPT], u32x4 (&xb)[UPT], const u32x4 &qwa, const u32x4 &qwb,
+                                             const u32x4 &kwa, const u32x4 &kwb, const u32x4 &cosv, const u32x4 &sinv,
+                                             float eps, int hq, int hl) {
+    constexpr int HPW = 64 / (D / 16);
 #pragma unroll
     for (int u = 0; u < UPT; ++u) {
         const int h0 = u * HPW;
@@ -583,9 +576,14 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
         norm_rotate<T, D, NEOX>(xa[u], xb[u], wa, wb, cosv, sinv, eps, oa, ob);
         xa[u] = oa, xb[u] = ob;
     }
+}
 
-    // ---- the writing half of the launch
-    while (__builtin_amdgcn_s_memrealtime() < entry + gate) __builtin_amdgcn_s_sleep(1);
+// The stores of a token: q_out rows, the K and V rows of its slot (dropped for a negative slot).
+template <typename T, int D, int UPT, bool KVFP8, int VN>
+__device__ __forceinline__ void token_store(const RopeArgs &a, uint32_t t, int64_t slot, const u32x4 (&xa)[UPT],
+                                            const u32x4 (&xb)[UPT], const u32x4 (&v)[VN], int hq, int hk, int hv, int lane) {
+    constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
+    const int sub = lane % LPH, hl = lane / LPH, heads_qk = hq + hk, v_chunks = hv * (D / 8);
     const bool slot_ok = slot >= 0;  // a negative slot: no place in the cache, the K and V rows are dropped
 #pragma unroll
     for (int u = 0; u < UPT; ++u) {
@@ -611,7 +609,7 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
         }
     }
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < VN; ++j) {
         const int c = lane + 64 * j;
         if (slot_ok && c < v_chunks) {
             const int64_t off = slot * hv * D + 8 * (int64_t)c;
@@ -622,6 +620,127 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
             } else {
                 *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(a.v_cache) + off) = v[j];
             }
+        }
+    }
+}
+
+constexpr int token_kernel_lds_bytes_per_wave(int upt) { return (2 * upt + 1) * 1024; }  // TWO: a token's units and 64 V chunks
+
+template <typename T, int D, bool NEOX, int UPT, bool KVFP8, int AXES, bool TWO>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
+rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num_tokens, uint32_t gate, int hq, int hk,
+                      int hv, uint32_t num_waves, int64_t ps_token, int64_t ps_axis, const RopeArgs rest) {
+    constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
+    constexpr int VN = TWO ? 1 : 2;  // V chunks per lane: the host admits 64 chunks per token with TWO, else 128
+    extern __shared__ __attribute__((aligned(16))) char token_lds[];  // TWO: 4 waves x token_kernel_lds_bytes_per_wave
+    const uint64_t entry = __builtin_amdgcn_s_memrealtime();
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t w = blockIdx.x * 4 + wave;
+    if (w >= num_waves) return;
+    const uint32_t t = w, t2 = w + num_waves;  // the wave's token(s)
+    const bool second = TWO && t2 < num_tokens;  // wave-uniform
+    const int lane = threadIdx.x & 63, sub = lane % LPH, hl = lane / LPH;
+    const int heads_qk = hq + hk, heads_all = heads_qk + hv, v_chunks = hv * (D / 8);
+    const uint16_t *token_in = static_cast<const uint16_t *>(qkv_in) + (int64_t)t * heads_all * D;
+
+    // ---- everything the wave reads, asked for at once (what needs only the leading parameters first)
+    u32x4 xa[UPT], xb[UPT], v[VN];
+#pragma unroll
+    for (int u = 0; u < UPT; ++u) {
+        const int head = min(u * HPW + hl, heads_qk - 1);  // lanes past the last head re-read it
+        const uint16_t *src = token_in + (int64_t)head * D;
+        xa[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 8 * sub));
+        xb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + HALF + 8 * sub));
+    }
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+        const int c = min(lane + 64 * j, v_chunks - 1);
+        v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(token_in + (int64_t)heads_qk * D + 8 * c));
+    }
+    uint32_t lds_base = 0;
+    if constexpr (TWO) {
+        lds_base = (uint32_t)(uintptr_t)token_lds + wave * (uint32_t)token_kernel_lds_bytes_per_wave(UPT);
+        if (second) {
+            const uint16_t *token2_in = static_cast<const uint16_t *>(qkv_in) + (int64_t)t2 * heads_all * D;
+#pragma unroll
+            for (int u = 0; u < UPT; ++u) {
+                const int head = min(u * HPW + hl, heads_qk - 1);
+                const uint16_t *src = token2_in + (int64_t)head * D;
+                lds_fill16(lds_base + (2 * u) * 1024u, src + 8 * sub);
+                lds_fill16(lds_base + (2 * u + 1) * 1024u, src + HALF + 8 * sub);
+            }
+            const int c = min(lane, v_chunks - 1);
+            lds_fill16(lds_base + (2 * UPT) * 1024u, token2_in + (int64_t)heads_qk * D + 8 * c);
+        }
+    }
+    // (positions: read as memory that no kernel of the launch writes, scalar loads whatever else the kernel contains)
+    int64_t p[3] = {0, 0, 0}, p2[3] = {0, 0, 0};
+#pragma unroll
+    for (int ax = 0; ax < AXES; ++ax) {
+        p[ax] = load_unchanging(positions + ax * ps_axis + (int64_t)t * ps_token);
+        if (second) p2[ax] = load_unchanging(positions + ax * ps_axis + (int64_t)t2 * ps_token);
+    }
+    // the rest of the arguments, fetched from the argument block behind the requests above (see rope_rms_kernel)
+    typedef const __attribute__((address_space(4))) RopeArgs *BlockPtr;
+    BlockPtr block = (BlockPtr)((const __attribute__((address_space(4))) char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                sizeof(TokenKernelLead));
+    asm volatile("" : "+s"(block));
+    RopeArgs a;
+    a.kv_loc = as_global(block->kv_loc);
+    a.qw = as_global(block->qw);
+    a.kw = as_global(block->kw);
+    a.cos_sin = as_global(block->cos_sin);
+    a.q_out = as_global(block->q_out);
+    a.k_cache = as_global(block->k_cache);
+    a.v_cache = as_global(block->v_cache);
+    a.eps = block->eps;
+    a.k_scale = block->k_scale;
+    a.v_scale = block->v_scale;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a.axis1[i] = AXES == 3 ? block->axis1[i] : 0u;
+        a.axis2[i] = AXES == 3 ? block->axis2[i] : 0u;
+    }
+    asm volatile("" ::"s"(a.kv_loc), "s"(a.qw), "s"(a.kw), "s"(a.cos_sin), "s"(a.q_out), "s"(a.k_cache), "s"(a.v_cache),
+                 "s"(a.eps), "s"(a.k_scale), "s"(a.v_scale));
+    const int64_t slot = load_unchanging(a.kv_loc + t);
+    const int64_t slot2 = second ? load_unchanging(a.kv_loc + t2) : -1;
+    const uint16_t *qw = static_cast<const uint16_t *>(a.qw), *kw = static_cast<const uint16_t *>(a.kw);
+    const u32x4 qwa = *reinterpret_cast<const u32x4 *>(qw + 8 * sub), qwb = *reinterpret_cast<const u32x4 *>(qw + HALF + 8 * sub);
+    const u32x4 kwa = *reinterpret_cast<const u32x4 *>(kw + 8 * sub), kwb = *reinterpret_cast<const u32x4 *>(kw + HALF + 8 * sub);
+    const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin);
+    u32x4 cosv, sinv, cosv2 = {0, 0, 0, 0}, sinv2 = {0, 0, 0, 0};
+    load_trig_by_axis<D, NEOX, AXES>(table, p[0], p[1], p[2], a.axis1, a.axis2, sub, cosv, sinv);
+    if (second) load_trig_by_axis<D, NEOX, AXES>(table, p2[0], p2[1], p2[2], a.axis1, a.axis2, sub, cosv2, sinv2);
+    // (the slots are asked for here and not where the rows are stored)
+    asm volatile("" ::"s"((uint32_t)slot), "s"((uint32_t)(slot >> 32)), "s"((uint32_t)slot2), "s"((uint32_t)(slot2 >> 32)));
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- norm and rotation of the first token, unit by unit, in place
+    token_rotate<T, D, NEOX, UPT>(xa, xb, qwa, qwb, kwa, kwb, cosv, sinv, a.eps, hq, hl);
+
+    // (the rotated rows are pinned down here, ahead of the wait: nothing ties the arithmetic to the clock, and the
+    // compiler otherwise moves it behind the wait, into the writing half)
+#pragma unroll
+    for (int u = 0; u < UPT; ++u) asm volatile("" ::"v"(xa[u]), "v"(xb[u]));
+
+    // ---- the writing half of the launch
+    while (__builtin_amdgcn_s_memrealtime() < entry + gate) __builtin_amdgcn_s_sleep(1);
+    // (the transfers into LDS are not loads the compiler knows of; they landed long ago, and with nothing else of
+    // the wave outstanding at this point the wait that says so to the hardware costs nothing)
+    if constexpr (TWO) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    token_store<T, D, UPT, KVFP8, VN>(a, t, slot, xa, xb, v, hq, hk, hv, lane);
+    if constexpr (TWO) {
+        if (second) {  // the second token takes the registers of the first
+            const char *mine = token_lds + wave * token_kernel_lds_bytes_per_wave(UPT) + lane * 16;
+#pragma unroll
+            for (int u = 0; u < UPT; ++u) {
+                xa[u] = *reinterpret_cast<const u32x4 *>(mine + (2 * u) * 1024);
+                xb[u] = *reinterpret_cast<const u32x4 *>(mine + (2 * u + 1) * 1024);
+            }
+            v[0] = *reinterpret_cast<const u32x4 *>(mine + (2 * UPT) * 1024);
+            token_rotate<T, D, NEOX, UPT>(xa, xb, qwa, qwb, kwa, kwb, cosv2, sinv2, a.eps, hq, hl);
+            token_store<T, D, UPT, KVFP8, VN>(a, t2, slot2, xa, xb, v, hq, hk, hv, lane);
         }
     }
 }
@@ -935,7 +1054,7 @@ int launch_2way_head_size(const TwoWayArgs &a, int64_t D, bool neox, unsigned ba
 int g_block_threads = 0;  // 0 = default
 int g_stream_rows = 0;    // output rows stored past the L2: 0 = built-in rule, 1 = never, 2 = always
 int g_merge_rows = 0;     // mRoPE rows merged on load where the sections allow: 0 = yes, 1 = never
-int g_token_waves = 0;    // one-wave-per-token kernel: 0 = built-in rule, 1 = never, 2 = wherever it fits
+int g_token_waves = 0;    // one-wave-per-token kernel: 0 = built-in rule, 1 = never, 2 = wherever it fits, 3 = likewise, two tokens per wave where that fits
 int g_token_gate = -1;    // its gate in ticks of 10 ns; -1 = from the bytes of the call
 int g_unit_gate = -1;     // gate of the kernel with one wave per unit: -1 = built-in rule, 0 = none, > 0 = ticks
 constexpr uint32_t kResidentUnits = 8192;  // waves of the one-wave-per-unit kernel the chip holds at once (8 per SIMD)
@@ -951,25 +1070,44 @@ struct RopePlan {
     uint32_t threads, blocks;  // workgroup size and count of the launch
     bool stream;               // q_out / K rows / in-place rows stored past the L2
     bool token_waves;          // the one-wave-per-token kernel
+    bool two_tokens;           // ... with two tokens per wave, the second through LDS
+    uint32_t token_wave_count; // its waves
     uint32_t gate;             // its gate: ticks of 10 ns before which no wave stores
     uint32_t unit_gate;        // the same for the kernel with one wave per unit (0 = none)
 };
 
 RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8) {
     RopePlan p{};
-    // One wave per token where the whole batch is resident at once and large enough for its traffic to matter:
-    // one position axis, head size 128, 4 or 5 units (25-40 Q and K heads) and at most 128 chunks of V per token.
+    // One wave per token (or per two) where the whole batch is resident at once and large enough for its traffic to
+    // matter: head size 128, 4 or 5 units (25-40 Q and K heads) and at most 128 chunks of V per token, a cache; with
+    // three position axes only where every aligned group of 8 frequencies takes one axis, and not with an fp8 cache.
     const int64_t read_bytes = 2 * (int64_t)a.num_tokens * (a.hq + a.hk + a.hv) * D;
-    const bool fits = axes == 1 && set_kv && D == 128 && a.units_per_token >= 4 && a.units_per_token <= 5 &&
-                      a.hv * (D / 8) <= 128 && a.hv > 0 && a.num_tokens <= kTokenWaveCapacity;
-    // ... and too large for the kernel above to hold all of its waves at once (more than 8192 units; below that the
-    // kernel above, gated, is ahead: 8.3 against 9.7 us at 1536 tokens of 32+8+8 heads; from there on this one is,
-    // 9.9 against 10.1 us at 1800 tokens, 10.3 against 11.1 at 2048, 13.6 against 14.8 at 3000, 16.6 against 17.3 at
-    // 3700, 17.4 against 18.8 at 4096; 28+4+4 heads: 11.0 against 11.9 us at 3000 tokens).  Not with an fp8 cache,
+    const bool shape = set_kv && D == 128 && a.units_per_token >= 4 && a.units_per_token <= 5 && a.hv * (D / 8) <= 128 &&
+                       a.hv > 0 && (axes == 1 || (axes == 3 && a.merge_rows && !kv_fp8));
+    const bool one = shape && a.num_tokens <= kTokenWaveCapacity;
+    // Two tokens per wave, the second through LDS (4 units and 64 V chunks per token: 9 KB of the 160 KB of a compute
+    // unit for each of its 16 waves), for up to twice that many tokens.
+    const bool two_shape = shape && a.units_per_token == 4 && a.hv * (D / 8) <= 64 && !kv_fp8 &&
+                           a.num_tokens <= 2 * kTokenWaveCapacity;
+    const bool two = two_shape && (g_token_waves == 3 || !one);
+    // ... and clearly too large for the kernel above to hold all of its waves at once (from 10240 units, five quarters
+    // of what it holds; below that the kernel above, gated, is ahead or level: 8.3 against 9.7 us at 1536 tokens of
+    // 32+8+8 heads, 9.1 against 9.5 at 2100 tokens of 28+4+4; from there on this one is: 32+8+8 heads 10.3 against
+    // 11.1 us at 2048 tokens, 13.6 against 14.8 at 3000, 16.6 against 17.3 at 3700, 16.2 against 18.2 at 4096; 28+4+4
+    // heads with three axes 10.0 against 11.7 us at 3000 tokens, 12.2 against 14.5 at 4096).  Not with an fp8 cache,
     // whose conversions lengthen the wave (32+8+8 heads: 15.7 against 14.4 us at 3000 tokens, 19.9 against 18.3 at 4096).
-    const bool large = a.total_units > kResidentUnits;
-    p.token_waves = fits && (g_token_waves == 2 || (g_token_waves == 0 && large && !kv_fp8));
-    const double gate = g_token_gate >= 0 ? (double)g_token_gate : (double)read_bytes / kGateBytesPerTick;
+    // With two tokens per wave only where the waves fill the SIMDs evenly, three or four on each: 19.1 against 20.3 us
+    // at 6144 tokens of 28+4+4 heads, 24.0 against 25.8 at 8192, but 22.8 against 23.1 at 7168 (three and a half
+    // waves per SIMD: the fuller ones set the time) and 17.9 against 17.5 at 5120.
+    const bool large = a.total_units >= kResidentUnits + kResidentUnits / 4;
+    const uint32_t waves2 = (a.num_tokens + 1) / 2, rounds2 = (waves2 + 1023) / 1024;
+    const bool even2 = rounds2 >= 3 && 100 * (uint64_t)waves2 >= 94 * (uint64_t)rounds2 * 1024;
+    const bool by_rule = g_token_waves == 0 && !kv_fp8 && (two ? even2 : large);
+    p.token_waves = (one || two) && (g_token_waves >= 2 || by_rule);
+    p.two_tokens = p.token_waves && two;
+    // (with two tokens per wave the full read time: 24.4 us at 8192 tokens of 28+4+4 heads with three axes, against 25.4
+    // with 0.95 of it, 24.8 with 1.05, 27.2 with 0.9 -- opening early, into the last reads, costs more than waiting)
+    const double gate = g_token_gate >= 0 ? (double)g_token_gate : (double)read_bytes / (two ? 70000.0 : kGateBytesPerTick);
     p.gate = (uint32_t)std::min(gate, 5000.0);
     // The kernel with one wave per unit gates its stores in the same way where its waves are all resident at once
     // (8192 of them, eight per SIMD, with one position axis) and fill at least half of that round; the gate is 0.85
@@ -1000,7 +1138,8 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     p.blocks = (a.total_units + units_per_block - 1) / units_per_block;
     if (p.token_waves) {
         p.threads = 256;
-        p.blocks = (a.num_tokens + 3) / 4;
+        p.token_wave_count = p.two_tokens ? (a.num_tokens + 1) / 2 : a.num_tokens;
+        p.blocks = (p.token_wave_count + 3) / 4;
         p.stream = true;
     }
     return p;
@@ -1012,16 +1151,25 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
     RopeArgs b = a;
     b.stream_rows = p.stream ? 1u : 0u;
     b.gate = p.unit_gate;
-    if constexpr (AXES == 1 && SETKV && D == 128) {
+    if constexpr (SETKV && D == 128 && (AXES == 1 || !KVFP8)) {
         if (p.token_waves) {
-            const uint32_t blocks = (a.num_tokens + 3) / 4;
-#define GPUK_LAUNCH_TOKEN(UPT)                                                                                         \
-    rope_rms_token_kernel<T, D, NEOX, UPT, KVFP8><<<blocks, 256, 0, stream>>>(a.qkv_in, a.positions, a.num_tokens, p.gate,   \
-                                                                            a.hq, a.hk, a.hv, a.ps_token, b)
-            switch (a.units_per_token) {
-                case 4: GPUK_LAUNCH_TOKEN(4); break;
-                case 5: GPUK_LAUNCH_TOKEN(5); break;
-                default: return GPUK_ERR_INTERNAL;
+#define GPUK_LAUNCH_TOKEN(UPT, TWO)                                                                                    \
+    rope_rms_token_kernel<T, D, NEOX, UPT, KVFP8, AXES, TWO>                                                           \
+        <<<p.blocks, 256, TWO ? 4 * token_kernel_lds_bytes_per_wave(UPT) : 0, stream>>>(                               \
+            a.qkv_in, a.positions, a.num_tokens, p.gate, a.hq, a.hk, a.hv, p.token_wave_count, a.ps_token, a.ps_axis, b)
+            if (p.two_tokens) {
+                if constexpr (!KVFP8) {
+                    if (a.units_per_token != 4) return GPUK_ERR_INTERNAL;
+                    GPUK_LAUNCH_TOKEN(4, true);
+                } else {
+                    return GPUK_ERR_INTERNAL;
+                }
+            } else {
+                switch (a.units_per_token) {
+                    case 4: GPUK_LAUNCH_TOKEN(4, false); break;
+                    case 5: GPUK_LAUNCH_TOKEN(5, false); break;
+                    default: return GPUK_ERR_INTERNAL;
+                }
             }
 #undef GPUK_LAUNCH_TOKEN
             return hip_status(hipGetLastError());
@@ -1213,6 +1361,7 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
     a.hq = (int)hq;
     a.hk = (int)hk;
     a.hv = (int)hv;
+    a.merge_rows = g_merge_rows == 1 ? 0u : 1u;  // (three axes: the answer is for sections that split at multiples of 8 frequencies)
     if (wide) {
         *workgroups = (int)((a.total_units + 3) / 4);
         *lanes = 256;
@@ -1223,7 +1372,7 @@ int rope_launch_shape(int64_t T, int64_t hq, int64_t hk, int64_t hv, int64_t D, 
     *workgroups = (int)p.blocks;
     *lanes = (int)p.threads;
     *streamed = p.stream ? 1 : 0;
-    *token_waves = p.token_waves ? 1 : 0;
+    *token_waves = p.token_waves ? (p.two_tokens ? 2 : 1) : 0;
     return GPUK_OK;
 }
 

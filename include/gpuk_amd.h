@@ -200,9 +200,11 @@ int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidden, int dtyp
 /*
  * The launch gpuk_rope_rms_set_kv (set_kv != 0) or gpuk_rope_rms (set_kv == 0) makes for a batch: the grid as
  * workgroups x lanes per workgroup; *streamed = 1 when the rotated rows are stored past the L2; *token_waves = 1 for
- * the kernel in which a wave of 64 lanes takes a whole token (batches the chip holds in one round), 0 for the one in
- * which it takes a group of heads of a token.  Computed on the host from the sizes and the tuning keys; the four
- * outputs are host pointers.  For reports.  Not part of the reference.
+ * the kernel in which a wave of 64 lanes takes a whole token (batches the chip holds in one round), 2 where it takes
+ * two tokens, the second through LDS, 0 for the kernel in which a wave takes a group of heads of a token.  Computed
+ * on the host from the sizes and the tuning keys (with three position axes: for sections that split at multiples of
+ * 8 frequencies, which the call itself checks); the four outputs are host pointers.  For reports.  Not part of the
+ * reference.
  */
 int gpuk_rope_rms_launch_shape(int64_t num_tokens, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
                                int64_t head_size, int n_axes, int dtype, int set_kv, int kv_dtype, int *workgroups,
@@ -223,7 +225,7 @@ int gpuk_increment_floats(float *data, int64_t n, void *stream);
  * "rope_block_threads" (64/128/256/512 lanes per workgroup of the rope kernel), "rope_stream_rows" (output rows of
  * the rope kernels stored past the L2: 1 never, 2 always), "rope_merge_rows" (1: never let the lanes of an mRoPE
  * token load their cos/sin pieces straight from the row of their axis), "rope_token_waves" (the kernel in which one
- * wave takes a whole token: 1 never, 2 wherever the shape fits it), "rope_token_gate" and "rope_unit_gate" (the
+ * wave takes a whole token: 1 never, 2 wherever the shape fits it, 3 likewise with two tokens per wave where that fits), "rope_token_gate" and "rope_unit_gate" (the
  * store gate of the two rope kernels, in ticks as above: -1 the built-in rule, 0 never).  The results do not depend
  * on any of them.  Unknown keys or values return GPUK_ERR_INVALID_ARG.  The settings are process-global plain
  * variables read at launch: set them from one thread while no other thread is launching.  Not part of the

@@ -327,18 +327,94 @@ def test_unit_kernel_store_gate_changes_no_bits(device, gate):
         capi.set_tuning("rope_token_waves", 0)
 
 
-def test_one_wave_per_token_kernel_by_rule(device):
-    """The launcher's rule takes that kernel where the other one could not hold all of its waves at once (more than
-    8192 groups of heads: 2049 tokens of 28+4 heads, not 2048) up to the 4096 tokens it holds itself, and not with an
-    fp8 cache; every choice meets the oracle."""
+TOKEN_WAVE_CASES_2 = [
+    # tokens, (hq, hk, hv), neox, sections (None: one position axis), two tokens per wave, fp16
+    (61, (28, 4, 4), True, [16, 24, 24], False, False),    # three axes, four units
+    (61, (28, 4, 4), False, [16, 24, 24], False, False),   # ... GPT-J pairs: a lane's two pieces may sit on two axes
+    (45, (32, 8, 8), True, [8, 24, 32], False, False),     # three axes, five units
+    (61, (28, 4, 4), True, None, True, False),             # two tokens per wave, an odd count: the last wave has one
+    (62, (28, 4, 4), True, [16, 24, 24], True, False),     # two tokens per wave and three axes
+    (37, (25, 7, 4), False, [32, 16, 16], True, False),    # a unit that mixes Q and K heads, GPT-J
+    (300, (30, 2, 1), True, [16, 24, 24], True, False),    # several workgroups, one V head
+    (33, (28, 4, 4), True, [16, 24, 24], True, True),      # fp16 activations
+    (1, (28, 4, 4), True, [16, 24, 24], True, False),      # a single token: one wave, no second token
+]
+
+
+@pytest.mark.parametrize("case", range(len(TOKEN_WAVE_CASES_2)))
+@pytest.mark.parametrize("gate", [-1, 700])
+def test_token_kernel_three_axes_and_two_tokens_per_wave(device, case, gate):
+    """The one-wave-per-token kernel with three position axes (sections that split at multiples of 8 frequencies: each
+    lane reads its cos/sin pieces from its axis's row) and with a second token per wave, which travels through LDS:
+    forced onto small batches, the oracle's bits and the same bits as the kernel with one wave per group of heads.
+    Tokens without a slot sit in the first and in the second half of the batch."""
     from gpuk_amd import capi
 
-    for tokens, fp8, expect in ((2048, False, False), (2049, False, True), (3500, False, True), (4096, False, True),
-                                (4097, False, False), (4000, True, False)):
-        groups, lanes, _, token_waves = capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 1, torch.bfloat16, True, fp8)
-        assert token_waves == expect and (not expect or (groups, lanes) == ((tokens + 3) // 4, 256)), (tokens, fp8, groups, lanes)
-        inp = make(tokens, 28, 128, True, seed=tokens + 1, fp8=fp8, hk=4, hv=4)
-        check_set_kv(inp, run_set_kv(inp, device), f"[rule T={tokens} fp8={fp8}]")
+    tokens, heads, neox, sections, two, fp16 = TOKEN_WAVE_CASES_2[case]
+    print(f"case token waves (2) {TOKEN_WAVE_CASES_2[case]} gate={gate}", flush=True)
+    inp = make(tokens, heads[0], 128, neox, seed=500 + case, mrope=sections is not None, hk=heads[1], hv=heads[2])
+    if sections is not None:
+        inp.mrope_section = sections
+    if fp16:
+        inp.qkv, inp.qw, inp.kw, inp.cos_sin = (t.to(torch.float16) for t in (inp.qkv, inp.qw, inp.kw, inp.cos_sin))
+        inp.kv_dtype = torch.float16
+    if tokens > 2:
+        inp.kv_loc[2], inp.kv_loc[tokens - 1] = -1, -7
+    n_axes = 3 if sections is not None else 1
+    try:
+        capi.set_tuning("rope_token_waves", 1)
+        base = run_set_kv(inp, device)
+        capi.set_tuning("rope_token_waves", 3 if two else 2)
+        capi.set_tuning("rope_token_gate", gate)
+        groups, lanes, _, token_waves = capi.rope_rms_launch_shape(tokens, *heads, 128, n_axes, inp.qkv.dtype, True, False)
+        waves = (tokens + 1) // 2 if two else tokens
+        assert token_waves == (2 if two else 1) and (groups, lanes) == ((waves + 3) // 4, 256), "the case must reach the kernel under test"
+        got = run_set_kv(inp, device)
+    finally:
+        capi.set_tuning("rope_token_waves", 0)
+        capi.set_tuning("rope_token_gate", -1)
+    raw = lambda t: t.cpu().contiguous().view(torch.uint8)
+    for name, a, b in zip(("q_out", "k_cache", "v_cache"), got[:3], base[:3]):
+        assert torch.equal(raw(a), raw(b)), f"{name}: the two kernels differ"
+    check_set_kv(inp, got, f"[token waves (2) {case}]")
+
+
+def test_token_kernel_leaves_other_sections_to_the_other_kernel(device):
+    """Sections that do not split at multiples of 8 frequencies, or the interleaved map, cannot take their cos/sin
+    pieces from one row per lane: even when the one-wave-per-token kernel is asked for, such calls run the other one
+    (and meet the oracle)."""
+    from gpuk_amd import capi
+
+    capi.set_tuning("rope_token_waves", 3)
+    try:
+        for sections, interleaved in (([24, 20, 20], False), ([16, 24, 24], True)):
+            inp = make(50, 28, 128, True, seed=77, mrope=True, interleaved=interleaved, hk=4, hv=4)
+            inp.mrope_section = sections
+            check_set_kv(inp, run_set_kv(inp, device), f"[sections {sections} interleaved={interleaved}]")
+    finally:
+        capi.set_tuning("rope_token_waves", 0)
+
+
+def test_one_wave_per_token_kernel_by_rule(device):
+    """The launcher's rule takes that kernel where the other one is clearly past what it holds at once (from 10240
+    groups of heads: 2560 tokens of 28+4 heads, not 2559) up to the 4096 tokens it holds itself; with two tokens per
+    wave where those waves fill the SIMDs evenly (6144 and 8192 tokens here, not 4097, 5000 or 8193); with one or three
+    position axes, and not with an fp8 cache.  Every choice meets the oracle."""
+    from gpuk_amd import capi
+
+    for tokens, mrope, fp8, expect in ((2559, False, False, 0), (2560, False, False, 1), (3500, True, False, 1),
+                                       (4096, False, False, 1), (4097, False, False, 0), (5000, True, False, 0),
+                                       (6144, True, False, 2), (8192, True, False, 2), (8192, False, False, 2),
+                                       (8193, False, False, 0), (4000, False, True, 0), (6144, False, True, 0)):
+        groups, lanes, _, token_waves = capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 3 if mrope else 1, torch.bfloat16, True, fp8)
+        waves = (tokens + 1) // 2 if expect == 2 else tokens
+        assert token_waves == expect and (not expect or (groups, lanes) == ((waves + 3) // 4, 256)), (tokens, fp8, groups, lanes)
+        inp = make(tokens, 28, 128, True, seed=tokens + 1, mrope=mrope, fp8=fp8, hk=4, hv=4)
+        if mrope:
+            inp.mrope_section = [16, 24, 24]
+        check_set_kv(inp, run_set_kv(inp, device), f"[rule T={tokens} mrope={mrope} fp8={fp8}]")
+    # 32+8+8 heads: five groups per token, one token per wave only
+    assert capi.rope_rms_launch_shape(4097, 32, 8, 8, 128)[3] == 0
 
 
 def test_batch_sizes_around_the_streaming_rule(device):
