@@ -185,6 +185,10 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
             if (!GATED && live[i]) store_stream(out + i * nthreads + tid, normed[i]);
         }
         if constexpr (GATED) {
+            // (the values to store are pinned down ahead of the wait: nothing ties the arithmetic to the clock, and the
+            // compiler otherwise moves it behind the wait)
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i) asm volatile("" ::"v"(normed[i]));
             while (__builtin_amdgcn_s_memrealtime() < entry + gate) __builtin_amdgcn_s_sleep(1);
 #pragma unroll
             for (int i = 0; i < NCHUNK; ++i)
@@ -258,6 +262,8 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
                 if (!GATED && live[i]) store_stream(out + i * nthreads + tid, codes[i]);
             }
             if constexpr (GATED) {
+#pragma unroll
+                for (int i = 0; i < NCHUNK; ++i) asm volatile("" ::"v"(codes[i]));  // computed ahead of the wait, as above
                 while (__builtin_amdgcn_s_memrealtime() < entry + gate) __builtin_amdgcn_s_sleep(1);
 #pragma unroll
                 for (int i = 0; i < NCHUNK; ++i)

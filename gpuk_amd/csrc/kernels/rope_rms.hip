@@ -339,8 +339,13 @@ struct RopeUnit {
 
         u32x4 oa, ob;
         norm_rotate<T, D, NEOX>(xa, xb, wa, wb, cosv, sinv, a.eps, oa, ob);
-        // batches whose waves are all resident at once: no store before the launch's reads are through
-        if constexpr (GATED) while (__builtin_amdgcn_s_memrealtime() < entry + a.gate) __builtin_amdgcn_s_sleep(1);
+        // batches whose waves are all resident at once: no store before the launch's reads are through (the rotated
+        // rows are pinned down ahead of the wait: nothing ties the arithmetic to the clock, and the compiler
+        // otherwise moves it behind the wait)
+        if constexpr (GATED) {
+            asm volatile("" ::"v"(oa), "v"(ob));
+            while (__builtin_amdgcn_s_memrealtime() < entry + a.gate) __builtin_amdgcn_s_sleep(1);
+        }
 
         // A negative slot marks a token that has no place in the cache (padding in a fixed-size decode batch): its Q
         // row is still produced, its K and V rows are dropped.  The reference would write out of bounds.
@@ -1110,18 +1115,23 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     const double gate = g_token_gate >= 0 ? (double)g_token_gate : (double)read_bytes / (two ? 70000.0 : kGateBytesPerTick);
     p.gate = (uint32_t)std::min(gate, 5000.0);
     // The kernel with one wave per unit gates its stores in the same way where its waves are all resident at once
-    // (8192 of them, eight per SIMD, with one position axis) and fill at least half of that round; the gate is 0.85
-    // of the read time at 7 TB/s, 0.7 of it with an fp8 cache (half the bytes to write) and then only from 0.7 of a
-    // round on.  Measured with a cache write: 64+8+8 heads, 16-bit cache, 7.1 against 7.8 us at 768 tokens, 7.8 against
-    // 8.9 at 900; fp8 cache, 7.4 against 7.9 us at 768 tokens, 8.2 against 8.7 at 900, but 5.9 against 5.8 at 512;
-    // 32+8+8 heads, 16-bit cache, 6.4 against 6.7 us at 1024 tokens, 8.3 against 9.1 at 1536; nothing to gain below
-    // half a round, 15-35 % slower one unit beyond a round, and 2 % at best with three position axes, whose
-    // instantiations hold seven waves per SIMD.
+    // (8192 of them, eight per SIMD, with one position axis) and fill at least half of that round.
+    // The gate is 1.15 to 1.2 times the read time at 7 TB/s (its waves enter over a few microseconds, and the gate
+    // counts from each wave's own entry); from two thirds of a round on the launch is made of four-wave workgroups
+    // whatever the head count, because 8192 single-wave workgroups take so long to place that the last waves' reads
+    // fall into the first waves' writes.  Measured (us, ungated single-wave workgroups / gated as chosen here): 32+8+8
+    // heads 6.6 / 5.9 at 1024 tokens, 7.9 / 7.0 at 1280, 9.1 / 7.7 at 1536, 9.5 / 8.0 at 1638; 64+8+8 heads 5.9 / 5.5 at
+    // 512 tokens, 7.4 / 6.6 at 700, 8.9 / 7.4 at 900; 28+4+4 heads 5.8 / 5.4 at 1024 tokens, 7.1 / 6.4 at 1536, 9.1 / 7.5
+    // at 2048.  With an fp8 cache (half the bytes to write) only from two thirds of a round on: 64+8+8 heads 7.6 / 7.4
+    // at 700 tokens, 8.8 / 8.1 at 900; 32+8+8 heads 9.3 / 8.8 at 1638.  Nothing to gain below half a round, 15-35 % slower
+    // one unit beyond a round, and 2 % at best with three position axes.
     p.unit_gate = 0;
+    const bool two_thirds = 3 * a.total_units > 2 * kResidentUnits;
+    const bool gated_by_rule = g_unit_gate < 0 && axes == 1 && set_kv && a.total_units <= kResidentUnits &&
+                               (kv_fp8 ? two_thirds : a.total_units >= kResidentUnits / 2);
+    const bool fuller = gated_by_rule && two_thirds;
     if (g_unit_gate > 0) p.unit_gate = (uint32_t)g_unit_gate;
-    else if (g_unit_gate < 0 && axes == 1 && set_kv && a.total_units <= kResidentUnits &&
-             a.total_units >= (kv_fp8 ? kResidentUnits * 7 / 10 : kResidentUnits / 2))
-        p.unit_gate = (uint32_t)std::min((kv_fp8 ? 0.7 : 0.85) * (double)read_bytes / 70000.0, 5000.0);
+    else if (gated_by_rule) p.unit_gate = (uint32_t)std::min((fuller ? 1.2 : 1.15) * (double)read_bytes / 70000.0, 5000.0);
     // bytes the call moves: every Q/K/V element in, Q (and K) elements out, the cache rows
     const int64_t elems_qk = (int64_t)a.num_tokens * (a.hq + a.hk) * D, elems_v = (int64_t)a.num_tokens * a.hv * D;
     const int64_t call_bytes = set_kv ? 2 * (elems_qk + elems_v) + 2 * (int64_t)a.num_tokens * a.hq * D +
@@ -1133,7 +1143,7 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     // CU's caches: 3-15 % ahead at 28+4 heads) and for large batches (1-3 % ahead from 4096 tokens on), single
     // waves for small batches of other head counts (2-6 % ahead at 64+8 heads with an fp8 cache up to 512 tokens,
     // within 1-3 % either way for 3, 5 and 6 units per token); 128 lanes is the slowest in most cases.
-    p.threads = g_block_threads ? (uint32_t)g_block_threads : (a.units_per_token % 4 == 0 || a.total_units > 8192 ? 256u : 64u);
+    p.threads = g_block_threads ? (uint32_t)g_block_threads : (a.units_per_token % 4 == 0 || a.total_units > 8192 || fuller ? 256u : 64u);
     const uint32_t units_per_block = p.threads / 64;
     p.blocks = (a.total_units + units_per_block - 1) / units_per_block;
     if (p.token_waves) {
