@@ -583,12 +583,24 @@ __device__ __forceinline__ void token_rotate(u32x4 (&xa)[UPT], u32x4 (&xb)[UPT],
     }
 }
 
-// The stores of a token: q_out rows, the K and V rows of its slot (dropped for a negative slot).
-template <typename T, int D, int UPT, bool KVFP8, int VN>
+// The stores of a token: q_out rows, the K and V rows of its slot (dropped for a negative slot); in place (!SETKV)
+// the rotated Q and K heads back where they came from.
+template <typename T, int D, int UPT, bool SETKV, bool KVFP8, int VN>
 __device__ __forceinline__ void token_store(const RopeArgs &a, uint32_t t, int64_t slot, const u32x4 (&xa)[UPT],
                                             const u32x4 (&xb)[UPT], const u32x4 (&v)[VN], int hq, int hk, int hv, int lane) {
     constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
     const int sub = lane % LPH, hl = lane / LPH, heads_qk = hq + hk, v_chunks = hv * (D / 8);
+    if constexpr (!SETKV) {
+#pragma unroll
+        for (int u = 0; u < UPT; ++u) {
+            const int head = u * HPW + hl;
+            if (head < heads_qk) {
+                uint16_t *dst = static_cast<uint16_t *>(a.qkv_out) + ((int64_t)t * (heads_qk + hv) + head) * D + 8 * sub;
+                store_pair<HALF * 2>(dst, xa[u], xb[u], true);
+            }
+        }
+        return;
+    }
     const bool slot_ok = slot >= 0;  // a negative slot: no place in the cache, the K and V rows are dropped
 #pragma unroll
     for (int u = 0; u < UPT; ++u) {
@@ -629,15 +641,15 @@ __device__ __forceinline__ void token_store(const RopeArgs &a, uint32_t t, int64
     }
 }
 
-constexpr int token_kernel_lds_bytes_per_wave(int upt) { return (2 * upt + 1) * 1024; }  // TWO: a token's units and 64 V chunks
+constexpr int token_kernel_lds_bytes_per_wave(int upt, bool set_kv) { return (2 * upt + (set_kv ? 1 : 0)) * 1024; }  // TWO: a token's units and 64 V chunks
 
-template <typename T, int D, bool NEOX, int UPT, bool KVFP8, int AXES, bool TWO>
+template <typename T, int D, bool NEOX, int UPT, bool SETKV, bool KVFP8, int AXES, bool TWO>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
 rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num_tokens, uint32_t gate, int hq, int hk,
                       int hv, uint32_t num_waves, int64_t ps_token, int64_t ps_axis, const RopeArgs rest) {
     constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
     constexpr int VN = TWO ? 1 : 2;  // V chunks per lane: the host admits 64 chunks per token with TWO, else 128
-    extern __shared__ __attribute__((aligned(16))) char token_lds[];  // TWO: 4 waves x token_kernel_lds_bytes_per_wave
+    extern __shared__ __attribute__((aligned(16))) char token_lds[];  // TWO: 4 waves x token_kernel_lds_bytes_per_wave()
     const uint64_t entry = __builtin_amdgcn_s_memrealtime();
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t w = blockIdx.x * 4 + wave;
@@ -657,14 +669,16 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
         xa[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 8 * sub));
         xb[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + HALF + 8 * sub));
     }
+    if constexpr (SETKV) {
 #pragma unroll
-    for (int j = 0; j < VN; ++j) {
-        const int c = min(lane + 64 * j, v_chunks - 1);
-        v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(token_in + (int64_t)heads_qk * D + 8 * c));
+        for (int j = 0; j < VN; ++j) {
+            const int c = min(lane + 64 * j, v_chunks - 1);
+            v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(token_in + (int64_t)heads_qk * D + 8 * c));
+        }
     }
     uint32_t lds_base = 0;
     if constexpr (TWO) {
-        lds_base = (uint32_t)(uintptr_t)token_lds + wave * (uint32_t)token_kernel_lds_bytes_per_wave(UPT);
+        lds_base = (uint32_t)(uintptr_t)token_lds + wave * (uint32_t)token_kernel_lds_bytes_per_wave(UPT, SETKV);
         if (second) {
             const uint16_t *token2_in = static_cast<const uint16_t *>(qkv_in) + (int64_t)t2 * heads_all * D;
 #pragma unroll
@@ -674,8 +688,10 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
                 lds_fill16(lds_base + (2 * u) * 1024u, src + 8 * sub);
                 lds_fill16(lds_base + (2 * u + 1) * 1024u, src + HALF + 8 * sub);
             }
-            const int c = min(lane, v_chunks - 1);
-            lds_fill16(lds_base + (2 * UPT) * 1024u, token2_in + (int64_t)heads_qk * D + 8 * c);
+            if constexpr (SETKV) {
+                const int c = min(lane, v_chunks - 1);
+                lds_fill16(lds_base + (2 * UPT) * 1024u, token2_in + (int64_t)heads_qk * D + 8 * c);
+            }
         }
     }
     // (positions: read as memory that no kernel of the launch writes, scalar loads whatever else the kernel contains)
@@ -691,25 +707,31 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
                                 sizeof(TokenKernelLead));
     asm volatile("" : "+s"(block));
     RopeArgs a;
-    a.kv_loc = as_global(block->kv_loc);
     a.qw = as_global(block->qw);
     a.kw = as_global(block->kw);
     a.cos_sin = as_global(block->cos_sin);
-    a.q_out = as_global(block->q_out);
-    a.k_cache = as_global(block->k_cache);
-    a.v_cache = as_global(block->v_cache);
     a.eps = block->eps;
-    a.k_scale = block->k_scale;
-    a.v_scale = block->v_scale;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         a.axis1[i] = AXES == 3 ? block->axis1[i] : 0u;
         a.axis2[i] = AXES == 3 ? block->axis2[i] : 0u;
     }
-    asm volatile("" ::"s"(a.kv_loc), "s"(a.qw), "s"(a.kw), "s"(a.cos_sin), "s"(a.q_out), "s"(a.k_cache), "s"(a.v_cache),
-                 "s"(a.eps), "s"(a.k_scale), "s"(a.v_scale));
-    const int64_t slot = load_unchanging(a.kv_loc + t);
-    const int64_t slot2 = second ? load_unchanging(a.kv_loc + t2) : -1;
+    int64_t slot = 0, slot2 = 0;
+    if constexpr (SETKV) {
+        a.kv_loc = as_global(block->kv_loc);
+        a.q_out = as_global(block->q_out);
+        a.k_cache = as_global(block->k_cache);
+        a.v_cache = as_global(block->v_cache);
+        a.k_scale = block->k_scale;
+        a.v_scale = block->v_scale;
+        asm volatile("" ::"s"(a.kv_loc), "s"(a.qw), "s"(a.kw), "s"(a.cos_sin), "s"(a.q_out), "s"(a.k_cache), "s"(a.v_cache),
+                     "s"(a.eps), "s"(a.k_scale), "s"(a.v_scale));
+        slot = load_unchanging(a.kv_loc + t);
+        slot2 = second ? load_unchanging(a.kv_loc + t2) : -1;
+    } else {
+        a.qkv_out = as_global(block->qkv_out);
+        asm volatile("" ::"s"(a.qw), "s"(a.kw), "s"(a.cos_sin), "s"(a.qkv_out), "s"(a.eps));
+    }
     const uint16_t *qw = static_cast<const uint16_t *>(a.qw), *kw = static_cast<const uint16_t *>(a.kw);
     const u32x4 qwa = *reinterpret_cast<const u32x4 *>(qw + 8 * sub), qwb = *reinterpret_cast<const u32x4 *>(qw + HALF + 8 * sub);
     const u32x4 kwa = *reinterpret_cast<const u32x4 *>(kw + 8 * sub), kwb = *reinterpret_cast<const u32x4 *>(kw + HALF + 8 * sub);
@@ -718,7 +740,8 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
     load_trig_by_axis<D, NEOX, AXES>(table, p[0], p[1], p[2], a.axis1, a.axis2, sub, cosv, sinv);
     if (second) load_trig_by_axis<D, NEOX, AXES>(table, p2[0], p2[1], p2[2], a.axis1, a.axis2, sub, cosv2, sinv2);
     // (the slots are asked for here and not where the rows are stored)
-    asm volatile("" ::"s"((uint32_t)slot), "s"((uint32_t)(slot >> 32)), "s"((uint32_t)slot2), "s"((uint32_t)(slot2 >> 32)));
+    if constexpr (SETKV)
+        asm volatile("" ::"s"((uint32_t)slot), "s"((uint32_t)(slot >> 32)), "s"((uint32_t)slot2), "s"((uint32_t)(slot2 >> 32)));
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- norm and rotation of the first token, unit by unit, in place
@@ -734,18 +757,18 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
     // (the transfers into LDS are not loads the compiler knows of; they landed long ago, and with nothing else of
     // the wave outstanding at this point the wait that says so to the hardware costs nothing)
     if constexpr (TWO) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    token_store<T, D, UPT, KVFP8, VN>(a, t, slot, xa, xb, v, hq, hk, hv, lane);
+    token_store<T, D, UPT, SETKV, KVFP8, VN>(a, t, slot, xa, xb, v, hq, hk, hv, lane);
     if constexpr (TWO) {
         if (second) {  // the second token takes the registers of the first
-            const char *mine = token_lds + wave * token_kernel_lds_bytes_per_wave(UPT) + lane * 16;
+            const char *mine = token_lds + wave * token_kernel_lds_bytes_per_wave(UPT, SETKV) + lane * 16;
 #pragma unroll
             for (int u = 0; u < UPT; ++u) {
                 xa[u] = *reinterpret_cast<const u32x4 *>(mine + (2 * u) * 1024);
                 xb[u] = *reinterpret_cast<const u32x4 *>(mine + (2 * u + 1) * 1024);
             }
-            v[0] = *reinterpret_cast<const u32x4 *>(mine + (2 * UPT) * 1024);
+            if constexpr (SETKV) v[0] = *reinterpret_cast<const u32x4 *>(mine + (2 * UPT) * 1024);
             token_rotate<T, D, NEOX, UPT>(xa, xb, qwa, qwb, kwa, kwb, cosv2, sinv2, a.eps, hq, hl);
-            token_store<T, D, UPT, KVFP8, VN>(a, t2, slot2, xa, xb, v, hq, hk, hv, lane);
+            token_store<T, D, UPT, SETKV, KVFP8, VN>(a, t2, slot2, xa, xb, v, hq, hk, hv, lane);
         }
     }
 }
@@ -1086,13 +1109,13 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     // One wave per token (or per two) where the whole batch is resident at once and large enough for its traffic to
     // matter: head size 128, 4 or 5 units (25-40 Q and K heads) and at most 128 chunks of V per token, a cache; with
     // three position axes only where every aligned group of 8 frequencies takes one axis, and not with an fp8 cache.
-    const int64_t read_bytes = 2 * (int64_t)a.num_tokens * (a.hq + a.hk + a.hv) * D;
-    const bool shape = set_kv && D == 128 && a.units_per_token >= 4 && a.units_per_token <= 5 && a.hv * (D / 8) <= 128 &&
-                       a.hv > 0 && (axes == 1 || (axes == 3 && a.merge_rows && !kv_fp8));
+    const int64_t read_bytes = 2 * (int64_t)a.num_tokens * (a.hq + a.hk + (set_kv ? a.hv : 0)) * D;
+    const bool shape = D == 128 && a.units_per_token >= 4 && a.units_per_token <= 5 &&
+                       (!set_kv || (a.hv * (D / 8) <= 128 && a.hv > 0)) && (axes == 1 || (axes == 3 && a.merge_rows && !kv_fp8));
     const bool one = shape && a.num_tokens <= kTokenWaveCapacity;
     // Two tokens per wave, the second through LDS (4 units and 64 V chunks per token: 9 KB of the 160 KB of a compute
     // unit for each of its 16 waves), for up to twice that many tokens.
-    const bool two_shape = shape && a.units_per_token == 4 && a.hv * (D / 8) <= 64 && !kv_fp8 &&
+    const bool two_shape = shape && a.units_per_token == 4 && (!set_kv || a.hv * (D / 8) <= 64) && !kv_fp8 &&
                            a.num_tokens <= 2 * kTokenWaveCapacity;
     const bool two = two_shape && (g_token_waves == 3 || !one);
     // ... and clearly too large for the kernel above to hold all of its waves at once (from 10240 units, five quarters
@@ -1104,7 +1127,11 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     // With two tokens per wave only where the waves fill the SIMDs evenly, three or four on each: 19.1 against 20.3 us
     // at 6144 tokens of 28+4+4 heads, 24.0 against 25.8 at 8192, but 22.8 against 23.1 at 7168 (three and a half
     // waves per SIMD: the fuller ones set the time) and 17.9 against 17.5 at 5120.
-    const bool large = a.total_units >= kResidentUnits + kResidentUnits / 4;
+    // (in place, with no V row and no scatter, the kernel above holds out a little longer: 9.0 against 9.5 us at 2048
+    // tokens of 32+8 heads, then 11.9 against 11.2 at 3000, 15.4 against 13.7 at 4096; 28+4 heads with three axes 10.7
+    // against 9.5 at 3000 tokens, 13.2 against 11.5 at 4096, 18.4 against 17.4 at 6144 and 23.2 against 21.6 at 8192 with
+    // two tokens per wave)
+    const bool large = a.total_units >= (set_kv ? kResidentUnits + kResidentUnits / 4 : kResidentUnits + 2 * kResidentUnits / 5);
     const uint32_t waves2 = (a.num_tokens + 1) / 2, rounds2 = (waves2 + 1023) / 1024;
     const bool even2 = rounds2 >= 3 && 100 * (uint64_t)waves2 >= 94 * (uint64_t)rounds2 * 1024;
     const bool by_rule = g_token_waves == 0 && !kv_fp8 && (two ? even2 : large);
@@ -1161,11 +1188,11 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
     RopeArgs b = a;
     b.stream_rows = p.stream ? 1u : 0u;
     b.gate = p.unit_gate;
-    if constexpr (SETKV && D == 128 && (AXES == 1 || !KVFP8)) {
+    if constexpr (D == 128 && (AXES == 1 || !KVFP8)) {
         if (p.token_waves) {
 #define GPUK_LAUNCH_TOKEN(UPT, TWO)                                                                                    \
-    rope_rms_token_kernel<T, D, NEOX, UPT, KVFP8, AXES, TWO>                                                           \
-        <<<p.blocks, 256, TWO ? 4 * token_kernel_lds_bytes_per_wave(UPT) : 0, stream>>>(                               \
+    rope_rms_token_kernel<T, D, NEOX, UPT, SETKV, KVFP8, AXES, TWO>                                                    \
+        <<<p.blocks, 256, TWO ? 4 * token_kernel_lds_bytes_per_wave(UPT, SETKV) : 0, stream>>>(                        \
             a.qkv_in, a.positions, a.num_tokens, p.gate, a.hq, a.hk, a.hv, p.token_wave_count, a.ps_token, a.ps_axis, b)
             if (p.two_tokens) {
                 if constexpr (!KVFP8) {

@@ -290,10 +290,11 @@ def test_rope_launch_shape_report():
     assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128) == (1024, 256, True, 1)
     # 4200 tokens do not: one wave per group of 8 Q/K heads, four waves a workgroup, streamed stores
     assert capi.rope_rms_launch_shape(4200, 32, 8, 8, 128) == (5250, 256, True, False)
-    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, set_kv=False) == (5120, 256, True, False)
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, set_kv=False) == (1024, 256, True, 1)   # in place too
+    assert capi.rope_rms_launch_shape(2048, 32, 8, 8, 128, set_kv=False) == (2560, 256, True, 0)
     # 8192 tokens of 28+4+4 heads: two tokens per wave, the second through LDS, still one round
     assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3) == (1024, 256, True, 2)
-    assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3, set_kv=False) == (8192, 256, True, 0)
+    assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3, set_kv=False) == (1024, 256, True, 2)
     assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (5120, 256, True, False)
     # a decode batch: through the L2; single waves unless a workgroup of four holds whole tokens
     assert capi.rope_rms_launch_shape(16, 28, 4, 4, 128) == (16, 256, False, False)

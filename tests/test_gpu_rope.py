@@ -370,13 +370,20 @@ def test_token_kernel_three_axes_and_two_tokens_per_wave(device, case, gate):
         waves = (tokens + 1) // 2 if two else tokens
         assert token_waves == (2 if two else 1) and (groups, lanes) == ((waves + 3) // 4, 256), "the case must reach the kernel under test"
         got = run_set_kv(inp, device)
+        # the in-place ops run the same kernel without the V row and the scatter
+        assert capi.rope_rms_launch_shape(tokens, *heads, 128, n_axes, inp.qkv.dtype, False, False)[3] == (2 if two else 1)
+        got_inplace = run_inplace(inp, device)
+        capi.set_tuning("rope_token_waves", 1)
+        base_inplace = run_inplace(inp, device)
     finally:
         capi.set_tuning("rope_token_waves", 0)
         capi.set_tuning("rope_token_gate", -1)
     raw = lambda t: t.cpu().contiguous().view(torch.uint8)
     for name, a, b in zip(("q_out", "k_cache", "v_cache"), got[:3], base[:3]):
         assert torch.equal(raw(a), raw(b)), f"{name}: the two kernels differ"
+    assert torch.equal(raw(got_inplace), raw(base_inplace)), "in place: the two kernels differ"
     check_set_kv(inp, got, f"[token waves (2) {case}]")
+    check_inplace(inp, got_inplace, f"[token waves (2) {case}, in place]")
 
 
 def test_token_kernel_leaves_other_sections_to_the_other_kernel(device):
@@ -415,6 +422,13 @@ def test_one_wave_per_token_kernel_by_rule(device):
         check_set_kv(inp, run_set_kv(inp, device), f"[rule T={tokens} mrope={mrope} fp8={fp8}]")
     # 32+8+8 heads: five groups per token, one token per wave only
     assert capi.rope_rms_launch_shape(4097, 32, 8, 8, 128)[3] == 0
+    # in place the other kernel holds out a little longer (to 11468 groups of heads)
+    for tokens, mrope, expect in ((2800, False, 0), (3000, True, 1), (8192, True, 2)):
+        assert capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 3 if mrope else 1, torch.bfloat16, False, False)[3] == expect
+        inp = make(tokens, 28, 128, True, seed=tokens + 2, mrope=mrope, hk=4, hv=4)
+        if mrope:
+            inp.mrope_section = [16, 24, 24]
+        check_inplace(inp, run_inplace(inp, device), f"[rule, in place, T={tokens} mrope={mrope}]")
 
 
 def test_batch_sizes_around_the_streaming_rule(device):
