@@ -503,10 +503,10 @@ rope_rms_kernel(const void *qkv_in, const int64_t *positions, uint32_t total_uni
 // together hold 8192 tokens of up to 32 Q and K heads and 4 V heads: twice the batch, still one round.
 // The arithmetic is norm_rotate's, as in the kernel above.
 constexpr uint32_t kTokenWaveCapacity = 4096;  // 4 waves per SIMD: the 100-odd registers a wave of this kernel takes
-// The gate: nine tenths of the time the launch's reads take at 7 TB/s, the rate of a read-only kernel on this part
-// (measured at 2900-4096 tokens of 28+4+4 and 32+8+8 heads: 3-7 % ahead of the kernel above with this gate, 2-4 %
-// with the full time, level or behind with 0.8 or 1.1 times it, and 6 % behind it with no gate at all).
-constexpr double kGateBytesPerTick = 70000.0 / 0.9;
+// The gate: 0.97 of the time the launch's reads take at 7 TB/s, the rate of a read-only kernel on this part (4096
+// tokens of 32+8+8 heads: 15.6-15.8 us with 0.95 to 1.0 of that time, 16.0 with 0.9, 17.0 with 0.85, 16.5 with 1.05,
+// 19-20 with no gate at all; the kernel above: 18.2).
+constexpr double kGateBytesPerTick = 70000.0 / 0.97;
 
 // The leading parameters of the kernel below as the argument segment lays them out; the block follows them.
 struct TokenKernelLead {
