@@ -1122,8 +1122,7 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     // of what it holds; below that the kernel above, gated, is ahead or level: 8.3 against 9.7 us at 1536 tokens of
     // 32+8+8 heads, 9.1 against 9.5 at 2100 tokens of 28+4+4; from there on this one is: 32+8+8 heads 10.3 against
     // 11.1 us at 2048 tokens, 13.6 against 14.8 at 3000, 16.6 against 17.3 at 3700, 16.2 against 18.2 at 4096; 28+4+4
-    // heads with three axes 10.0 against 11.7 us at 3000 tokens, 12.2 against 14.5 at 4096).  Not with an fp8 cache,
-    // whose conversions lengthen the wave (32+8+8 heads: 15.7 against 14.4 us at 3000 tokens, 19.9 against 18.3 at 4096).
+    // heads with three axes 10.0 against 11.7 us at 3000 tokens, 12.2 against 14.5 at 4096).
     // With two tokens per wave only where the waves fill the SIMDs evenly, three or four on each: 19.1 against 20.3 us
     // at 6144 tokens of 28+4+4 heads, 24.0 against 25.8 at 8192, but 22.8 against 23.1 at 7168 (three and a half
     // waves per SIMD: the fuller ones set the time) and 17.9 against 17.5 at 5120.
@@ -1134,7 +1133,11 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     const bool large = a.total_units >= (set_kv ? kResidentUnits + kResidentUnits / 4 : kResidentUnits + 2 * kResidentUnits / 5);
     const uint32_t waves2 = (a.num_tokens + 1) / 2, rounds2 = (waves2 + 1023) / 1024;
     const bool even2 = rounds2 >= 3 && 100 * (uint64_t)waves2 >= 94 * (uint64_t)rounds2 * 1024;
-    const bool by_rule = g_token_waves == 0 && !kv_fp8 && (two ? even2 : large);
+    // (with an fp8 cache the conversions lengthen the wave and the gate hardly matters; one token per wave is still
+    // ahead once the batch is large: 28+4+4 heads 10.8 against 11.9 us at 3000 tokens, 13.3 against 14.2 at 4096; 32+8+8
+    // heads 16.8 against 17.6 at 4096, level at 3000, behind at 2560)
+    const bool large_fp8 = a.total_units >= (a.units_per_token == 4 ? kResidentUnits + kResidentUnits / 4 : 7 * kResidentUnits / 4);
+    const bool by_rule = g_token_waves == 0 && (two ? even2 : (kv_fp8 ? large_fp8 : large));
     p.token_waves = (one || two) && (g_token_waves >= 2 || by_rule);
     p.two_tokens = p.token_waves && two;
     // (with two tokens per wave the full read time: 24.4 us at 8192 tokens of 28+4+4 heads with three axes, against 25.4
@@ -1142,20 +1145,22 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     const double gate = g_token_gate >= 0 ? (double)g_token_gate : (double)read_bytes / (two ? 70000.0 : kGateBytesPerTick);
     p.gate = (uint32_t)std::min(gate, 5000.0);
     // The kernel with one wave per unit gates its stores in the same way where its waves are all resident at once
-    // (8192 of them, eight per SIMD, with one position axis) and fill at least half of that round.
+    // (8192 of them, eight per SIMD) and fill at least half of that round.
     // The gate is 1.15 to 1.2 times the read time at 7 TB/s (its waves enter over a few microseconds, and the gate
     // counts from each wave's own entry); from two thirds of a round on the launch is made of four-wave workgroups
     // whatever the head count, because 8192 single-wave workgroups take so long to place that the last waves' reads
     // fall into the first waves' writes.  Measured (us, ungated single-wave workgroups / gated as chosen here): 32+8+8
     // heads 6.6 / 5.9 at 1024 tokens, 7.9 / 7.0 at 1280, 9.1 / 7.7 at 1536, 9.5 / 8.0 at 1638; 64+8+8 heads 5.9 / 5.5 at
     // 512 tokens, 7.4 / 6.6 at 700, 8.9 / 7.4 at 900; 28+4+4 heads 5.8 / 5.4 at 1024 tokens, 7.1 / 6.4 at 1536, 9.1 / 7.5
-    // at 2048.  With an fp8 cache (half the bytes to write) only from two thirds of a round on: 64+8+8 heads 7.6 / 7.4
-    // at 700 tokens, 8.8 / 8.1 at 900; 32+8+8 heads 9.3 / 8.8 at 1638.  Nothing to gain below half a round, 15-35 % slower
-    // one unit beyond a round, and 2 % at best with three position axes.
+    // at 2048.  With an fp8 cache (half the bytes to write) or three position axes only from two thirds of a round on:
+    // 64+8+8 heads, fp8, 7.6 / 7.4 at 700 tokens, 8.8 / 8.1 at 900; 28+4+4 heads with three axes 7.2 / 6.6 at 1536 tokens,
+    // 9.2 / 7.7 at 2048 (5.5 / 5.7 at 1024).  The in-place ops alike: 32+8 heads 5.9 / 5.5 at 1024 tokens, 7.3 / 6.4 at 1400,
+    // 8.2 / 7.0 at 1638; 28+4 heads with three axes 6.8 / 6.2 at 1536 tokens, 8.5 / 7.1 at 2048.  Nothing to gain below
+    // half a round, 15-35 % slower one unit beyond a round.
     p.unit_gate = 0;
     const bool two_thirds = 3 * a.total_units > 2 * kResidentUnits;
-    const bool gated_by_rule = g_unit_gate < 0 && axes == 1 && set_kv && a.total_units <= kResidentUnits &&
-                               (kv_fp8 ? two_thirds : a.total_units >= kResidentUnits / 2);
+    const bool gated_by_rule = g_unit_gate < 0 && a.total_units <= kResidentUnits &&
+                               (two_thirds || (axes == 1 && !kv_fp8 && a.total_units >= kResidentUnits / 2));
     const bool fuller = gated_by_rule && two_thirds;
     if (g_unit_gate > 0) p.unit_gate = (uint32_t)g_unit_gate;
     else if (gated_by_rule) p.unit_gate = (uint32_t)std::min((fuller ? 1.2 : 1.15) * (double)read_bytes / 70000.0, 5000.0);
@@ -1217,13 +1222,8 @@ int launch_one(const RopeArgs &a, hipStream_t stream) {
     rope_rms_kernel<T, D, NEOX, AXES, SETKV, KVFP8, GATED><<<p.blocks, p.threads, 0, stream>>>(                         \
         a.qkv_in, a.positions, a.total_units, a.units_per_token, a.upt_magic, a.hq, a.hk,                               \
         (uint32_t)a.hv | (log2_waves << 24), a.ps_token, a.ps_axis, b)
-    if constexpr (AXES == 1 && SETKV) {  // the only launches the rule gates
-        if (b.gate) GPUK_LAUNCH_UNITS(true);
-        else GPUK_LAUNCH_UNITS(false);
-    } else {
-        b.gate = 0;
-        GPUK_LAUNCH_UNITS(false);
-    }
+    if (b.gate) GPUK_LAUNCH_UNITS(true);
+    else GPUK_LAUNCH_UNITS(false);
 #undef GPUK_LAUNCH_UNITS
     return hip_status(hipGetLastError());
 }

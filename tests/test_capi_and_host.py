@@ -295,7 +295,8 @@ def test_rope_launch_shape_report():
     # 8192 tokens of 28+4+4 heads: two tokens per wave, the second through LDS, still one round
     assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3) == (1024, 256, True, 2)
     assert capi.rope_rms_launch_shape(8192, 28, 4, 4, 128, n_axes=3, set_kv=False) == (1024, 256, True, 2)
-    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (5120, 256, True, False)
+    assert capi.rope_rms_launch_shape(4096, 32, 8, 8, 128, kv_fp8=True) == (1024, 256, True, 1)
+    assert capi.rope_rms_launch_shape(2560, 32, 8, 8, 128, kv_fp8=True) == (3200, 256, True, 0)   # an fp8 cache: later
     # a decode batch: through the L2; single waves unless a workgroup of four holds whole tokens
     assert capi.rope_rms_launch_shape(16, 28, 4, 4, 128) == (16, 256, False, False)
     assert capi.rope_rms_launch_shape(16, 40, 8, 8, 128, kv_fp8=True) == (96, 64, False, False)

@@ -309,9 +309,8 @@ def test_one_wave_per_token_kernel(device, case, gate):
 @pytest.mark.parametrize("gate", [0, 1, 400])
 def test_unit_kernel_store_gate_changes_no_bits(device, gate):
     """The kernel with one wave per group of heads holds its stores back, where all of its waves are resident at
-    once (one position axis, a cache write), until the launch's reads are through.  Forced onto small batches: no
-    gate, the shortest, 4 us -- the oracle's bits every time; with three position axes or in place the key is
-    ignored and the bits are the oracle's too."""
+    once, until the launch's reads are through.  Forced onto small batches: no gate, the shortest, 4 us -- the oracle's
+    bits every time, with one and three position axes, a 16-bit and an fp8 cache, and in place."""
     from gpuk_amd import capi
 
     print(f"case unit kernel gate {gate}", flush=True)
@@ -406,13 +405,13 @@ def test_one_wave_per_token_kernel_by_rule(device):
     """The launcher's rule takes that kernel where the other one is clearly past what it holds at once (from 10240
     groups of heads: 2560 tokens of 28+4 heads, not 2559) up to the 4096 tokens it holds itself; with two tokens per
     wave where those waves fill the SIMDs evenly (6144 and 8192 tokens here, not 4097, 5000 or 8193); with one or three
-    position axes, and not with an fp8 cache.  Every choice meets the oracle."""
+    position axes; with an fp8 cache one token per wave only.  Every choice meets the oracle."""
     from gpuk_amd import capi
 
     for tokens, mrope, fp8, expect in ((2559, False, False, 0), (2560, False, False, 1), (3500, True, False, 1),
                                        (4096, False, False, 1), (4097, False, False, 0), (5000, True, False, 0),
                                        (6144, True, False, 2), (8192, True, False, 2), (8192, False, False, 2),
-                                       (8193, False, False, 0), (4000, False, True, 0), (6144, False, True, 0)):
+                                       (8193, False, False, 0), (2500, False, True, 0), (4000, False, True, 1), (6144, False, True, 0)):
         groups, lanes, _, token_waves = capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 3 if mrope else 1, torch.bfloat16, True, fp8)
         waves = (tokens + 1) // 2 if expect == 2 else tokens
         assert token_waves == expect and (not expect or (groups, lanes) == ((waves + 3) // 4, 256)), (tokens, fp8, groups, lanes)
