@@ -947,43 +947,76 @@ struct TwoWayArgs {
     uint32_t stream;  // 1: the output rows are stored past the L2 (calls that move more than a few MB)
 };
 
+// The leading parameters of the kernel below as the argument segment lays them out; the block follows them.
+struct TwoWayKernelLead {
+    const void *q0, *k0, *q1, *k1;
+    uint32_t tokens0, tokens1, heads_q, heads_k, stream;
+    uint32_t pad_;
+};
+static_assert(sizeof(TwoWayKernelLead) == 56 && sizeof(TwoWayKernelLead) % alignof(TwoWayArgs) == 0, "offset of the block");
+
+// As in rope_rms_kernel, what a wave needs to find and request its activations -- the four input pointers, the token
+// and head counts -- are leading scalar parameters that arrive in scalar registers at launch; segment bounds and
+// row counts are products and sums of those, not loads.  (With everything in the argument block and the per-segment
+// values picked by index, a wave went through five dependent fetches of the block before its first request.)  The
+// block (weights, tables, outputs, the division constants) is fetched behind the activations, in one batch.
 template <typename T, int D, bool NEOX>
-__global__ void __launch_bounds__(256) rope_rms_2way_kernel(const TwoWayArgs a) {
+__global__ void __launch_bounds__(256)
+rope_rms_2way_kernel(const void *q0, const void *k0, const void *q1, const void *k1, uint32_t tokens0, uint32_t tokens1,
+                     uint32_t heads_q, uint32_t heads_k, uint32_t stream, const TwoWayArgs rest) {
     constexpr int LPH = D / 16, HPW = 64 / LPH, HALF = D / 2;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t unit = blockIdx.x * (blockDim.x >> 6) + wave;
-    if (unit >= a.unit_end[3]) return;
-    const int seg = (unit >= a.unit_end[0]) + (unit >= a.unit_end[1]) + (unit >= a.unit_end[2]);  // wave-uniform
-    const uint32_t unit_in_seg = unit - (seg ? a.unit_end[seg - 1] : 0u);
+    const uint32_t unit = blockIdx.x * 4 + wave;
+    const uint32_t rows0 = tokens0 * heads_q, rows1 = tokens0 * heads_k, rows2 = tokens1 * heads_q, rows3 = tokens1 * heads_k;
+    const uint32_t end0 = (rows0 + HPW - 1) / HPW, end1 = end0 + (rows1 + HPW - 1) / HPW, end2 = end1 + (rows2 + HPW - 1) / HPW,
+                   end3 = end2 + (rows3 + HPW - 1) / HPW;
+    if (unit >= end3) return;
+    const int seg = (unit >= end0) + (unit >= end1) + (unit >= end2);  // wave-uniform
+    const uint32_t unit_in_seg = unit - (seg == 0 ? 0u : seg == 1 ? end0 : seg == 2 ? end1 : end2);
     const int kind = seg & 1, stream_id = seg >> 1;  // q|k, stream 0|1
-    const uint32_t heads = a.heads[kind], rows = a.rows[seg];
+    const uint32_t heads = kind ? heads_k : heads_q;
+    const uint32_t rows = seg == 0 ? rows0 : seg == 1 ? rows1 : seg == 2 ? rows2 : rows3;
+    const void *in = seg == 0 ? q0 : seg == 1 ? k0 : seg == 2 ? q1 : k1;
     const int batch = blockIdx.y;
 
     const int lane = threadIdx.x & 63, sub = lane % LPH, hl = lane / LPH;
     const uint32_t row_raw = unit_in_seg * HPW + hl;
     const bool active = row_raw < rows;
     const uint32_t row = min(row_raw, rows - 1);  // (token, head) flattened inside the segment
-    const uint32_t token = a.heads_magic[kind] ? __umulhi(row, a.heads_magic[kind]) : row;
-    const uint32_t head = row - token * heads;
 
     const int c0 = 8 * sub, c1 = HALF + 8 * sub;
-    const uint16_t *src = static_cast<const uint16_t *>(a.in[seg]) + ((int64_t)batch * rows + row) * D;
+    const uint16_t *src = static_cast<const uint16_t *>(in) + ((int64_t)batch * rows + row) * D;
     const u32x4 xa = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c0));
     const u32x4 xb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c1));
-    const uint16_t *wsrc = static_cast<const uint16_t *>(a.w[seg]);
+
+    typedef const __attribute__((address_space(4))) TwoWayArgs *BlockPtr;
+    BlockPtr block = (BlockPtr)((const __attribute__((address_space(4))) char *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                sizeof(TwoWayKernelLead));
+    asm volatile("" : "+s"(block));
+    const void *w0 = as_global(block->w[0]), *w1 = as_global(block->w[1]), *w2 = as_global(block->w[2]), *w3 = as_global(block->w[3]);
+    const void *table0 = as_global(block->cos_sin[0]), *table1 = as_global(block->cos_sin[1]);
+    void *out_q = as_global(block->out[0]), *out_k = as_global(block->out[1]);
+    const uint32_t magic_q = block->heads_magic[0], magic_k = block->heads_magic[1];
+    const float eps = block->eps;
+    asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(w3), "s"(table0), "s"(table1), "s"(out_q), "s"(out_k), "s"(magic_q),
+                 "s"(magic_k), "s"(eps));
+    const uint32_t magic = kind ? magic_k : magic_q;
+    const uint32_t token = magic ? __umulhi(row, magic) : row;
+    const uint32_t head = row - token * heads;
+    const uint16_t *wsrc = static_cast<const uint16_t *>(seg == 0 ? w0 : seg == 1 ? w1 : seg == 2 ? w2 : w3);
     const u32x4 wa = *reinterpret_cast<const u32x4 *>(wsrc + c0);
     const u32x4 wb = *reinterpret_cast<const u32x4 *>(wsrc + c1);
-    const uint16_t *table = static_cast<const uint16_t *>(a.cos_sin[stream_id]) + (int64_t)token * D;
+    const uint16_t *table = static_cast<const uint16_t *>(stream_id ? table1 : table0) + (int64_t)token * D;
     const u32x4 cosv = load_trig<D, NEOX>(table, sub);
     const u32x4 sinv = load_trig<D, NEOX>(table + HALF, sub);
     __builtin_amdgcn_sched_barrier(0);
 
     u32x4 oa, ob;
-    norm_rotate<T, D, NEOX>(xa, xb, wa, wb, cosv, sinv, a.eps, oa, ob);
+    norm_rotate<T, D, NEOX>(xa, xb, wa, wb, cosv, sinv, eps, oa, ob);
     if (active) {
-        const int64_t out_token = (int64_t)batch * (a.tokens0 + a.tokens1) + (stream_id ? a.tokens0 : 0) + token;
-        uint16_t *dst = static_cast<uint16_t *>(a.out[kind]) + (out_token * heads + head) * D;
-        store_pair<HALF * 2>(dst + c0, oa, ob, a.stream != 0);
+        const int64_t out_token = (int64_t)batch * (tokens0 + tokens1) + (stream_id ? tokens0 : 0u) + token;
+        uint16_t *dst = static_cast<uint16_t *>(kind ? out_k : out_q) + (out_token * heads + head) * D;
+        store_pair<HALF * 2>(dst + c0, oa, ob, stream != 0);
     }
 }
 
@@ -1046,8 +1079,12 @@ __global__ void __launch_bounds__(256) rope_rms_2way_wide_kernel(const TwoWayArg
 template <typename T, int D>
 int launch_2way(const TwoWayArgs &a, bool neox, unsigned batch, hipStream_t stream) {
     const dim3 grid((a.unit_end[3] + 3) / 4, batch);
-    if (neox) rope_rms_2way_kernel<T, D, true><<<grid, 256, 0, stream>>>(a);
-    else rope_rms_2way_kernel<T, D, false><<<grid, 256, 0, stream>>>(a);
+#define GPUK_LAUNCH_2WAY(NEOX)                                                                                         \
+    rope_rms_2way_kernel<T, D, NEOX><<<grid, 256, 0, stream>>>(a.in[0], a.in[1], a.in[2], a.in[3], (uint32_t)a.tokens0,  \
+                                                               (uint32_t)a.tokens1, a.heads[0], a.heads[1], a.stream, a)
+    if (neox) GPUK_LAUNCH_2WAY(true);
+    else GPUK_LAUNCH_2WAY(false);
+#undef GPUK_LAUNCH_2WAY
     return hip_status(hipGetLastError());
 }
 
