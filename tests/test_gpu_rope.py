@@ -401,6 +401,50 @@ def test_token_kernel_leaves_other_sections_to_the_other_kernel(device):
         capi.set_tuning("rope_token_waves", 0)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_token_kernel_random_shapes(device, seed):
+    """Seeded random shapes for the one-wave-per-token kernel, forced onto small batches: 25-40 Q and K heads in any
+    split (also none of one kind), 1-8 V heads, NeoX or GPT-J, one axis or three (random sections that split at
+    multiples of 8 frequencies), a 16-bit or fp8 cache, one or two tokens per wave, with a cache write and in place;
+    the same bits as the kernel with one wave per group of heads every time, and the oracle's bits."""
+    from gpuk_amd import capi
+
+    g = torch.Generator().manual_seed(9000 + seed)
+    rnd = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    two = bool(rnd(0, 1))
+    heads_qk = rnd(25, 32) if two else rnd(25, 40)
+    hq = rnd(0, heads_qk)
+    hk = heads_qk - hq
+    hv = rnd(1, 4) if two else rnd(1, 8)
+    tokens = rnd(1, 700)
+    neox = bool(rnd(0, 1))
+    mrope = bool(rnd(0, 1))
+    fp8 = (not mrope) and (not two) and bool(rnd(0, 1))
+    print(f"case token fuzz seed={seed} T={tokens} heads=({hq},{hk},{hv}) neox={neox} mrope={mrope} fp8={fp8} two={two}", flush=True)
+    inp = make(tokens, hq, 128, neox, seed=9100 + seed, mrope=mrope, fp8=fp8, hk=hk, hv=hv)
+    if mrope:
+        a = 8 * rnd(0, 8)
+        b = 8 * rnd(0, (64 - a) // 8)
+        inp.mrope_section = [a, b, 64 - a - b]
+    if tokens > 3:
+        inp.kv_loc[rnd(0, tokens - 1)] = -1
+    n_axes = 3 if mrope else 1
+    try:
+        capi.set_tuning("rope_token_waves", 1)
+        base, base_inplace = run_set_kv(inp, device), run_inplace(inp, device)
+        capi.set_tuning("rope_token_waves", 3 if two else 2)
+        assert capi.rope_rms_launch_shape(tokens, hq, hk, hv, 128, n_axes, inp.qkv.dtype, True, fp8)[3] == (2 if two else 1)
+        got, got_inplace = run_set_kv(inp, device), run_inplace(inp, device)
+    finally:
+        capi.set_tuning("rope_token_waves", 0)
+    raw = lambda t: t.cpu().contiguous().view(torch.uint8)
+    for name, x, y in zip(("q_out", "k_cache", "v_cache"), got[:3], base[:3]):
+        assert torch.equal(raw(x), raw(y)), f"{name}: the two kernels differ"
+    assert torch.equal(raw(got_inplace), raw(base_inplace)), "in place: the two kernels differ"
+    check_set_kv(inp, got, f"[token fuzz {seed}]")
+    check_inplace(inp, got_inplace, f"[token fuzz {seed}, in place]")
+
+
 def test_one_wave_per_token_kernel_by_rule(device):
     """The launcher's rule takes that kernel where the other one is clearly past what it holds at once (from 10240
     groups of heads: 2560 tokens of 28+4 heads, not 2559) up to the 4096 tokens it holds itself; with two tokens per
@@ -613,12 +657,16 @@ def test_negative_slots_and_colliding_slots(device, fp8):
     assert bool(k_close.all()), f"K pieces not from any colliding token: {(~k_close).nonzero().flatten().tolist()}"
 
 
-def test_rope_kernel_replayed_from_a_graph(device):
+@pytest.mark.parametrize("token_waves", [0, 2, 3])
+def test_rope_kernel_replayed_from_a_graph(device, token_waves):
     """The mRoPE + KV-write op recorded into a HIP graph: every replay, with fresh inputs copied into the captured
-    buffers and eager work in between, equals the eager call on the same inputs."""
+    buffers and eager work in between, equals the eager call on the same inputs -- with the kernel the rule picks,
+    and with the one-wave-per-token kernel forced, one and two tokens per wave (the latter holds data in LDS and
+    both time their stores by the wall clock)."""
     import gpuk_amd as gpuk
     from gpuk_amd import capi
 
+    capi.set_tuning("rope_token_waves", token_waves)
     T, hq, hk, hv, D = 300, 28, 4, 4, 128
     inp = make(T, hq, D, True, seed=71, mrope=True, hk=hk, hv=hv)
     inp.mrope_section = ALIGNED_SECTIONS[D]
@@ -658,3 +706,4 @@ def test_rope_kernel_replayed_from_a_graph(device):
             assert torch.equal(raw(kc[loc]), raw(k2[loc])) and torch.equal(raw(vc[loc]), raw(v2[loc])), f"replay {rep}: cache rows"
     finally:
         torch.cuda.synchronize()
+        capi.set_tuning("rope_token_waves", 0)
