@@ -136,6 +136,10 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
     // left to itself the compiler fetches them where they are first used, after the first barrier, and every wave of
     // the row then waits there for the scalar cache (0.1-0.15 us of a decode-sized call).
     asm volatile("" ::"s"(hidden_f), "s"(rcp_hidden), "s"(hidden_pow2), "s"(eps), "s"(fp8_max), "s"(rcp_fp8_max));
+    // ... and so is the static scale, which the kernel only reads (asked for here, needed in phase 3: fetched where it
+    // is first used it put a round trip through the scalar cache between the last two phases)
+    float static_scale = 0.f;
+    if constexpr (QUANT == GPUK_QUANT_FP8_STATIC) static_scale = *(const __attribute__((address_space(4))) float *)scale_io;
     GPUK_STAMP(1);          // every load issued
     GPUK_STAMP_DRAINED(2);  // ... and landed
 
@@ -155,6 +159,7 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
         if (!GATED && live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
     }
     float sumsq[1] = {ss0 + ss1};
+    if constexpr (QUANT == GPUK_QUANT_FP8_STATIC) asm volatile("" ::"s"(static_scale));  // (it has arrived by now)
     GPUK_STAMP(3);  // residual stored, the lane's squares summed
     block_allreduce<SumOp, 1>(sumsq, s_sum, num_waves);
     __builtin_amdgcn_s_setprio(0);
@@ -235,7 +240,7 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
                 scale = amax[0] == 0.f ? 1.f : amax[0] / fp8_max;
             if (tid == 0) scale_io[row] = scale;
         } else {
-            scale = scale_io[0];
+            scale = static_scale;
         }
 
         // ---- phase 3: code = e4m3fn(clamp(n2 / scale)), 8 codes per chunk.  With the dynamic scale every value is
