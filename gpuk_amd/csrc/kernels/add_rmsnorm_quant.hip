@@ -533,6 +533,14 @@ int g_row_group_shift = -1;  // -1 = heuristic, else log2 of the run of consecut
 int g_gate = -1;             // store gate in ticks of 10 ns: -1 = built-in rule, 0 = none, > 0 = that many
 constexpr int kComputeUnits = 256;  // MI355X
 
+// Rows resident at once, chip-wide, with `threads` lanes per row and `nchunk` chunks per lane: 2048 lanes per compute
+// unit, and with four chunks per lane the gated kernel's 70 registers allow seven waves per SIMD, not eight.
+int64_t resident_rows(int threads, int nchunk) {
+    int per_cu = 2048 / threads;
+    if (nchunk >= 4) per_cu = std::min(per_cu, 28 / (threads / 64));
+    return (int64_t)kComputeUnits * per_cu;
+}
+
 // The store gate of a launch of 16-bit rows: for batches whose workgroups are all resident at once (2048 lanes per
 // compute unit) the time their reads take at 7 TB/s, the rate of a read-only kernel on this part, plus a twentieth;
 // 0 (stores as soon as they are ready) for larger batches, whose later workgroups read while earlier ones write
@@ -540,11 +548,12 @@ constexpr int kComputeUnits = 256;  // MI355X
 // 768, 9.0 against 11.7 at 1024 (gate 1.0-1.1 times the read time; 10.2 with 0.9, 9.6 with 1.2), nothing gained and
 // 0.1 us lost below a quarter of a round; at 4096 elements 6.2 against 7.7 us at 1024 rows, 10.2 against 12.4 at 2048; 20-45 % slower where the
 // batch does not fit one round.
-uint32_t store_gate(int64_t tokens, int64_t hidden, int threads) {
+uint32_t store_gate(int64_t tokens, int64_t hidden, int threads, int nchunk) {
     if (g_gate >= 0) return (uint32_t)g_gate;
-    const int64_t resident_rows = (int64_t)kComputeUnits * (2048 / threads);
-    if (tokens > resident_rows || 4 * tokens < resident_rows) return 0;
-    const double ticks = 1.05 * (double)(4 * tokens * hidden) / 70000.0;  // 70,000 bytes per tick of 10 ns
+    const int64_t resident = resident_rows(threads, nchunk);
+    if (tokens > resident || 4 * tokens < resident) return 0;
+    // (four chunks per lane: the shape pick_shape takes to hold in one round what two chunks per lane cannot)
+    const double ticks = (nchunk >= 4 ? 1.08 : 1.05) * (double)(4 * tokens * hidden) / 70000.0;  // 70,000 bytes per tick of 10 ns
     return (uint32_t)std::min(ticks, 5000.0);
 }
 
@@ -556,7 +565,6 @@ uint32_t store_gate(int64_t tokens, int64_t hidden, int threads) {
 void pick_shape(int64_t tokens, int chunks_per_row, int *threads, int *nchunk) {
     auto fits = [&](int n) { return (int64_t)n * kMaxThreads >= chunks_per_row; };
     int n;
-    (void)tokens;  // the same shape serves one row and thousands: measured at 7168 elements from 1 to 4096 rows
     if (g_force_nchunk) {
         n = g_force_nchunk;
     } else {
@@ -564,6 +572,16 @@ void pick_shape(int64_t tokens, int chunks_per_row, int *threads, int *nchunk) {
         const int lanes1 = round_up(chunks_per_row, 64), lanes2 = round_up((chunks_per_row + 1) / 2, 64);
         n = (2 * lanes2 > lanes1 && lanes1 <= kMaxThreads) ? 1 : 2;
         while (n < 8 && chunks_per_row > kMaxThreads * n) n *= 2;
+        // A batch that two chunks per lane cannot hold in one round but four can (half the lanes per row, so up to
+        // 1792 rows of 7168 or 8192 elements instead of 1024) takes four: one round, with the store gate, against two
+        // rounds of mixed reads and writes.  7168 elements: 10.8 against 12.8 us at 1100 rows, 10.9 against 14.3 at
+        // 1280, 13.0 against 16.2 at 1536, 14.3 against 17.5 at 1700; 8192 elements: 12.4 against 15.5 us at 1280 rows,
+        // 16.3 against 18.7 at 1700.  (Held to 64 registers for an eighth wave per SIMD the kernel spills, and its
+        // 2048 rows take 17.9 us against 20.4; not done: the spill costs 1 us at 1700 rows.)
+        if (n == 2 && !g_force_threads) {
+            const int t2 = round_up((chunks_per_row + 1) / 2, 64), t4 = round_up((chunks_per_row + 3) / 4, 64);
+            if (tokens > resident_rows(t2, 2) && tokens <= resident_rows(t4, 4)) n = 4;
+        }
     }
     while (n < 8 && !fits(n)) n *= 2;
     if (!fits(n)) {
@@ -596,7 +614,7 @@ int launch(const void *x, const void *residual_in, const void *gamma, void *resi
     const float rcp_hidden = 1.0f / hf;
     const int hidden_pow2 = (hidden & (hidden - 1)) == 0;
     const float rcp_fp8_max = (fp8_max == 448.0f || fp8_max == 240.0f) ? 1.0f / fp8_max : 0.0f;
-    const uint32_t gate = store_gate(tokens, hidden, threads);
+    const uint32_t gate = store_gate(tokens, hidden, threads, nchunk);
     // Runs of 64 rows per XCD: measured +1.1 % for 16 KiB rows (8192 rows); neutral or 1-10 % slower for every other
     // row size tried (2, 3, 4, 8, 10, 14, 32 KiB) and for fewer rows, hence the narrow rule.
     const int64_t row_bytes = hidden * 2;
@@ -729,7 +747,7 @@ extern "C" int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *re
     auto ro = static_cast<u32x4 *>(residual_out);
     auto co = static_cast<u32x2 *>(codes);
     const dim3 grid((unsigned)tokens);
-    const uint32_t gate = store_gate(tokens, hidden, threads);
+    const uint32_t gate = store_gate(tokens, hidden, threads, nchunk);
     const uint32_t shape = (uint32_t)threads | ((uint32_t)group_shift << 16);
     switch (nchunk) {
         case 1: add_rmsnorm_quant_traffic_only<1><<<grid, threads, 0, s>>>(xs, rs, chunks, remap_end, shape, gate, ro, co, scale); break;
