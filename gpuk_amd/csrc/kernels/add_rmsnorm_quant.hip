@@ -79,7 +79,7 @@ __device__ __attribute__((noinline)) u32x2 codes_by_division(f32x8 n, float scal
 // (true for every power-of-two row and for 7168 elements; it removes a sixth of the kernel's instructions, which is
 // what a decode-sized batch waits for: with at most one row per compute unit the run time is the row's arithmetic).
 template <typename T, int NCHUNK, int QUANT, bool EXACT, bool GATED>
-__global__ void __launch_bounds__(kMaxThreads)
+__global__ void __launch_bounds__(kMaxThreads) __attribute__((amdgpu_waves_per_eu(GATED && NCHUNK <= 4 ? 8 : 4)))
 add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_row, int remap_end,
                        uint32_t lanes_and_shift, uint32_t gate, const u32x4 *__restrict__ gamma, u32x4 *residual_out,
                        void *norm_out, float *__restrict__ scale_io, float hidden_f, float rcp_hidden, int hidden_pow2,
@@ -158,6 +158,12 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
         }
         if (!GATED && live[i]) store_stream(residual_out + row_base + i * nthreads + tid, xv[i]);
     }
+    if constexpr (GATED && NCHUNK == 4) {  // (the packed residual is what stays in registers, not the sums it was rounded from)
+#pragma unroll
+        for (int i = 0; i < NCHUNK; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(xv[i][j]));
+    }
     float sumsq[1] = {ss0 + ss1};
     if constexpr (QUANT == GPUK_QUANT_FP8_STATIC) asm volatile("" ::"s"(static_scale));  // (it has arrived by now)
     GPUK_STAMP(3);  // residual stored, the lane's squares summed
@@ -209,17 +215,28 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
     } else {
         // the normed row stays in fp32 registers, every value already rounded to the 16-bit type.
         // v_max3_f32 drops NaNs where the reference's amax propagates them: they are tracked apart
-        float nv[NCHUNK][8];
+        // (kPacked, the gated four-chunk form: as 16-bit pairs instead, half the registers, so that eight waves fit a
+        // SIMD with the residual kept for the gate as well; unpacked again in phase 3)
+        constexpr bool kPacked = GATED && NCHUNK == 4;
+        float nv[kPacked ? 1 : NCHUNK][8];
+        uint32_t nw[kPacked ? NCHUNK : 1][4];
         float m0 = 0.f, m1 = 0.f;
         bool any_nan = false;
 #pragma unroll
         for (int i = 0; i < NCHUNK; ++i) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float lo = P::round(P::lo(gv[i][j]) * P::round(P::lo(xv[i][j]) * rstd));
-                const float hi = P::round(P::hi(gv[i][j]) * P::round(P::hi(xv[i][j]) * rstd));
-                nv[i][2 * j] = lo;
-                nv[i][2 * j + 1] = hi;
+                float lo, hi;
+                if constexpr (kPacked) {
+                    nw[i][j] = P::pack(P::lo(gv[i][j]) * P::round(P::lo(xv[i][j]) * rstd), P::hi(gv[i][j]) * P::round(P::hi(xv[i][j]) * rstd));
+                    lo = P::lo(nw[i][j]);
+                    hi = P::hi(nw[i][j]);
+                } else {
+                    lo = P::round(P::lo(gv[i][j]) * P::round(P::lo(xv[i][j]) * rstd));
+                    hi = P::round(P::hi(gv[i][j]) * P::round(P::hi(xv[i][j]) * rstd));
+                    nv[i][2 * j] = lo;
+                    nv[i][2 * j + 1] = hi;
+                }
                 if constexpr (QUANT == GPUK_QUANT_FP8_DYNAMIC) {
                     if (j & 1) m1 = max3_abs(m1, lo, hi);
                     else m0 = max3_abs(m0, lo, hi);
@@ -249,6 +266,12 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
         // division gives for infinite and NaN numerators.
         constexpr bool kDynamic = QUANT == GPUK_QUANT_FP8_DYNAMIC;
         u32x2 *out = reinterpret_cast<u32x2 *>(norm_out) + row_base;
+        if constexpr (kPacked) {  // (or the compiler keeps phase 2's unpacked copies alive instead)
+#pragma unroll
+            for (int i = 0; i < NCHUNK; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(nw[i][j]));
+        }
         // (the scale is the same in every lane; deciding by ballot tells the compiler so, and the common path is
         // laid out as straight-line code with the other one out of the way)
         if (__builtin_expect(__builtin_amdgcn_ballot_w64(!scale_in_fast_range(scale)) == 0, 1)) {
@@ -261,7 +284,12 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
             for (int i = 0; i < NCHUNK; ++i) {
                 float q[8];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) q[j] = kDynamic ? div_by_rcp_finite(nv[i][j], scale, rcp) : div_by_rcp(nv[i][j], scale, rcp);
+                for (int j = 0; j < 8; ++j) {
+                    float n;
+                    if constexpr (kPacked) n = (j & 1) ? P::hi(nw[i][j >> 1]) : P::lo(nw[i][j >> 1]);
+                    else n = nv[i][j];
+                    q[j] = kDynamic ? div_by_rcp_finite(n, scale, rcp) : div_by_rcp(n, scale, rcp);
+                }
                 if constexpr (!kDynamic) clamp8_sym(q, fp8_max);
                 codes[i] = u32x2{cvt4_e4m3fn(q[0], q[1], q[2], q[3]), cvt4_e4m3fn(q[4], q[5], q[6], q[7])};
                 if (!GATED && live[i]) store_stream(out + i * nthreads + tid, codes[i]);
@@ -286,7 +314,12 @@ add_rmsnorm_quant_rows(const u32x4 *x, const u32x4 *residual_in, int chunks_per_
             // (unrolled like the common path: a runtime index into the register arrays would move them to scratch)
 #pragma unroll
             for (int i = 0; i < NCHUNK; ++i) {
-                const f32x8 n = {nv[i][0], nv[i][1], nv[i][2], nv[i][3], nv[i][4], nv[i][5], nv[i][6], nv[i][7]};
+                f32x8 n;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if constexpr (kPacked) n[j] = (j & 1) ? P::hi(nw[i][j >> 1]) : P::lo(nw[i][j >> 1]);
+                    else n[j] = nv[i][j];
+                }
                 const u32x2 codes = codes_by_division(n, scale, fp8_max);
                 if (live[i]) store_stream(out + i * nthreads + tid, codes);
             }
@@ -534,11 +567,11 @@ int g_gate = -1;             // store gate in ticks of 10 ns: -1 = built-in rule
 constexpr int kComputeUnits = 256;  // MI355X
 
 // Rows resident at once, chip-wide, with `threads` lanes per row and `nchunk` chunks per lane: 2048 lanes per compute
-// unit, and with four chunks per lane the gated kernel's 70 registers allow seven waves per SIMD, not eight.
+// unit, eight waves per SIMD, which the gated instantiations of up to four chunks per lane are compiled for
+// (amdgpu_waves_per_eu: at most 64 registers); with eight chunks per lane, up to 128 registers, half of that.
 int64_t resident_rows(int threads, int nchunk) {
-    int per_cu = 2048 / threads;
-    if (nchunk >= 4) per_cu = std::min(per_cu, 28 / (threads / 64));
-    return (int64_t)kComputeUnits * per_cu;
+    const int waves_per_cu = nchunk >= 8 ? 16 : 32;
+    return (int64_t)kComputeUnits * (waves_per_cu / (threads / 64));
 }
 
 // The store gate of a launch of 16-bit rows: for batches whose workgroups are all resident at once (2048 lanes per
@@ -573,11 +606,11 @@ void pick_shape(int64_t tokens, int chunks_per_row, int *threads, int *nchunk) {
         n = (2 * lanes2 > lanes1 && lanes1 <= kMaxThreads) ? 1 : 2;
         while (n < 8 && chunks_per_row > kMaxThreads * n) n *= 2;
         // A batch that two chunks per lane cannot hold in one round but four can (half the lanes per row, so up to
-        // 1792 rows of 7168 or 8192 elements instead of 1024) takes four: one round, with the store gate, against two
+        // 2048 rows of 7168 or 8192 elements instead of 1024) takes four: one round, with the store gate, against two
         // rounds of mixed reads and writes.  7168 elements: 10.8 against 12.8 us at 1100 rows, 10.9 against 14.3 at
         // 1280, 13.0 against 16.2 at 1536, 14.3 against 17.5 at 1700; 8192 elements: 12.4 against 15.5 us at 1280 rows,
-        // 16.3 against 18.7 at 1700.  (Held to 64 registers for an eighth wave per SIMD the kernel spills, and its
-        // 2048 rows take 17.9 us against 20.4; not done: the spill costs 1 us at 1700 rows.)
+        // 16.3 against 18.7 at 1700.  (That form keeps the normed row as 16-bit pairs between its last two phases:
+        // with it in fp32 the kernel took 70 registers, seven waves per SIMD, 1792 rows.)
         if (n == 2 && !g_force_threads) {
             const int t2 = round_up((chunks_per_row + 1) / 2, 64), t4 = round_up((chunks_per_row + 3) / 4, 64);
             if (tokens > resident_rows(t2, 2) && tokens <= resident_rows(t4, 4)) n = 4;

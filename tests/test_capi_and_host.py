@@ -261,11 +261,11 @@ def test_launch_shape_report():
 
     assert capi.add_rmsnorm_quant_launch_shape(8192, 8192) == (512, 2)
     assert capi.add_rmsnorm_quant_launch_shape(512, 7168) == (448, 2)
-    # 1025-1792 rows of 7168: too many for one round at two chunks per lane, not at four (half the lanes per row)
+    # 1025-2048 rows of 7168: too many for one round at two chunks per lane, not at four (half the lanes per row)
     assert capi.add_rmsnorm_quant_launch_shape(1024, 7168) == (448, 2)
     assert capi.add_rmsnorm_quant_launch_shape(1025, 7168) == (256, 4)
-    assert capi.add_rmsnorm_quant_launch_shape(1792, 8192) == (256, 4)
-    assert capi.add_rmsnorm_quant_launch_shape(1793, 8192) == (512, 2)
+    assert capi.add_rmsnorm_quant_launch_shape(2048, 8192) == (256, 4)
+    assert capi.add_rmsnorm_quant_launch_shape(2049, 8192) == (512, 2)
     assert capi.add_rmsnorm_quant_launch_shape(1, 4096) == (256, 2)
     lanes, chunks = capi.add_rmsnorm_quant_launch_shape(4, 65600 * 2)    # rows that do not stay in registers
     assert chunks == 0 and lanes % 64 == 0

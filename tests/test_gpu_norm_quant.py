@@ -215,17 +215,21 @@ def test_store_gate_changes_no_bits(device, gate):
         capi.set_tuning("norm_quant_gate", -1)
 
 
-@pytest.mark.parametrize("tokens,hidden", [(1025, 7168), (1700, 7168), (1792, 8192), (1793, 8192), (3000, 4096)])
-def test_batches_between_one_and_two_rounds(device, tokens, hidden):
-    """Batches that two chunks per lane cannot hold in one round and four can (1025-1792 rows of 7168 or 8192
+@pytest.mark.parametrize("tokens,hidden,dtype", [(1025, 7168, torch.bfloat16), (1700, 7168, torch.bfloat16),
+                                                 (2048, 8192, torch.bfloat16), (2049, 8192, torch.bfloat16),
+                                                 (3000, 4096, torch.bfloat16), (1700, 5120, torch.bfloat16),
+                                                 (2048, 7168, torch.float16), (2000, 5120, torch.float16)])
+def test_batches_between_one_and_two_rounds(device, tokens, hidden, dtype):
+    """Batches that two chunks per lane cannot hold in one round and four can (1025-2048 rows of 7168 or 8192
     elements) run four chunks per lane on half the lanes, with the store gate; one row more runs the usual shape.
-    The oracle's bits either way, in every quant mode."""
+    Rows of 5120 elements are the masked form of that kernel (160 lanes' chunks on 192 lanes).  The oracle's bits
+    either way, in every quant mode."""
     from gpuk_amd import capi
 
-    lanes, chunks = capi.add_rmsnorm_quant_launch_shape(tokens, hidden, torch.bfloat16)
-    print(f"case between rounds {tokens}x{hidden}: {lanes} lanes x {chunks} chunks", flush=True)
-    assert chunks == (2 if (tokens, hidden) == (1793, 8192) else 4)
-    inp = workloads.norm_quant_inputs(tokens, hidden, seed=tokens, res_sigma=2.0, outlier_frac=0.01)
+    lanes, chunks = capi.add_rmsnorm_quant_launch_shape(tokens, hidden, dtype)
+    print(f"case between rounds {tokens}x{hidden} {dtype}: {lanes} lanes x {chunks} chunks", flush=True)
+    assert chunks == (2 if (tokens, hidden) == (2049, 8192) else 4)
+    inp = workloads.norm_quant_inputs(tokens, hidden, seed=tokens, res_sigma=2.0, outlier_frac=0.01, dtype=dtype)
     for quant in (0, 1, 3):
         st = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
         check(inp, quant, run_capi(inp, quant, device, static_scale=st), static_scale=st, tag=f"[{tokens}x{hidden} q{quant}]")
