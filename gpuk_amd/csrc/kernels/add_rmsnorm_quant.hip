@@ -564,14 +564,20 @@ int g_force_nchunk = 0;   // 0 = heuristic; set through gpuk_set_tuning for swee
 int g_force_threads = 0;  // 0 = heuristic
 int g_row_group_shift = -1;  // -1 = heuristic, else log2 of the run of consecutive rows an XCD takes (0 = one row)
 int g_gate = -1;             // store gate in ticks of 10 ns: -1 = built-in rule, 0 = none, > 0 = that many
+int g_pieces = 0;            // launches per call: 0 = built-in rule, 1 = always one, 2 = two wherever each half fits one round
 constexpr int kComputeUnits = 256;  // MI355X
 
 // Rows resident at once, chip-wide, with `threads` lanes per row and `nchunk` chunks per lane: 2048 lanes per compute
 // unit, eight waves per SIMD, which the gated instantiations of up to four chunks per lane are compiled for
 // (amdgpu_waves_per_eu: at most 64 registers); with eight chunks per lane, up to 128 registers, half of that.
+// Measured exception: of workgroups of 5 or 10 waves a compute unit takes 25 or 20 waves' worth, not 30 (1408 rows of
+// 5120 elements, 5.5 per compute unit, run no faster gated than ungated, 1280 run 22 % faster; likewise 640 and 512
+// rows of 10240), where 3, 6, 7, 9, 11-16 waves fill it as counted (30, 30, 28, 27, ... waves).
 int64_t resident_rows(int threads, int nchunk) {
-    const int waves_per_cu = nchunk >= 8 ? 16 : 32;
-    return (int64_t)kComputeUnits * (waves_per_cu / (threads / 64));
+    const int waves = threads / 64;
+    int waves_per_cu = nchunk >= 8 ? 16 : 32;
+    if (waves == 5 || waves == 10) waves_per_cu = std::min(waves_per_cu, waves == 5 ? 25 : 20);
+    return (int64_t)kComputeUnits * (waves_per_cu / waves);
 }
 
 // The store gate of a launch of 16-bit rows: for batches whose workgroups are all resident at once (2048 lanes per
@@ -628,9 +634,46 @@ void pick_shape(int64_t tokens, int chunks_per_row, int *threads, int *nchunk) {
     *threads = t;
 }
 
+// Launches per call.  A batch of more than one round of workgroups and at most two runs as two launches of half the
+// rows, each a round of its own with the store gate: a read phase and a write phase twice over instead of two rounds
+// that mix the directions.
+int launches_for(int64_t tokens, int chunks_per_row) {
+    if (g_pieces == 1 || g_force_nchunk || g_force_threads || chunks_per_row > 2 * kMaxThreads) return 1;
+    const int64_t round = resident_rows(round_up((chunks_per_row + 3) / 4, 64), 4);
+    if (tokens <= round || tokens > 2 * round) return 1;
+    if (g_pieces == 2) return 2;
+    return 10 * tokens >= 11 * round ? 2 : 1;
+}
+
+// Rows of the first launch: the whole batch, or of two pieces the first, a whole number of rows per compute unit (half
+// of what the batch needs, rounded down), so that neither piece pays for a partly filled last row of workgroups twice.
+int64_t first_piece(int64_t tokens, int chunks_per_row) {
+    if (launches_for(tokens, chunks_per_row) == 1) return tokens;
+    return (tokens + kComputeUnits - 1) / kComputeUnits / 2 * kComputeUnits;
+}
+
+template <typename T, int QUANT>
+int launch_rows(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
+                float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream);
+
 template <typename T, int QUANT>
 int launch(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
            float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream) {
+    const int64_t piece = first_piece(tokens, (int)(hidden / 8));
+    for (int64_t first = 0; first < tokens; first = first ? tokens : piece) {
+        const int64_t in_bytes = first * hidden * 2, out_bytes = first * hidden * (QUANT == GPUK_QUANT_NONE ? 2 : 1);
+        const int rc = launch_rows<T, QUANT>(static_cast<const char *>(x) + in_bytes, static_cast<const char *>(residual_in) + in_bytes,
+                                             gamma, static_cast<char *>(residual_out) + in_bytes, static_cast<char *>(norm_out) + out_bytes,
+                                             QUANT == GPUK_QUANT_FP8_DYNAMIC ? scale + first : scale, first ? tokens - first : piece,
+                                             hidden, eps, fp8_max, stream);
+        if (rc != GPUK_OK) return rc;
+    }
+    return GPUK_OK;
+}
+
+template <typename T, int QUANT>
+int launch_rows(const void *x, const void *residual_in, const void *gamma, void *residual_out, void *norm_out,
+                float *scale, int64_t tokens, int64_t hidden, float eps, float fp8_max, hipStream_t stream) {
     const int chunks = (int)(hidden / 8);
     int threads, nchunk;
     pick_shape(tokens, chunks, &threads, &nchunk);
@@ -754,6 +797,7 @@ void set_norm_quant_tuning(int key, int value) {
     if (key == 1) g_force_threads = value;
     if (key == 5) g_row_group_shift = value;
     if (key == 6) g_gate = value;
+    if (key == 7) g_pieces = value;
 }
 
 }  // namespace gpuk
@@ -769,6 +813,14 @@ extern "C" int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *re
     if (!x || !residual_in || !residual_out || !codes || !scale) return GPUK_ERR_INVALID_ARG;
     if (!aligned16(x) || !aligned16(residual_in) || !aligned16(residual_out) || !aligned8(codes)) return GPUK_ERR_MISALIGNED;
     const int chunks = (int)(hidden / 8);
+    if (const int64_t piece = first_piece(tokens, chunks); piece < tokens) {  // two launches where the op takes two
+        const int rc = gpuk_add_rmsnorm_quant_traffic_only(x, residual_in, residual_out, codes, scale, piece, hidden, stream);
+        if (rc != GPUK_OK) return rc;
+        const int64_t wide = piece * hidden * 2, narrow = piece * hidden;
+        return gpuk_add_rmsnorm_quant_traffic_only(static_cast<const char *>(x) + wide, static_cast<const char *>(residual_in) + wide,
+                                                   static_cast<char *>(residual_out) + wide, static_cast<char *>(codes) + narrow,
+                                                   scale + piece, tokens - piece, hidden, stream);
+    }
     int threads, nchunk;
     pick_shape(tokens, chunks, &threads, &nchunk);
     if (nchunk == 0) return GPUK_ERR_UNSUPPORTED;  // rows that do not stay in registers
@@ -802,7 +854,7 @@ extern "C" int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidde
         pick_wide_shape((int)(hidden / 4), dtype == GPUK_DTYPE_F64, lanes_per_row, chunks_per_lane);
         return GPUK_OK;
     }
-    pick_shape(tokens, (int)(hidden / 8), lanes_per_row, chunks_per_lane);
+    pick_shape(first_piece(tokens, (int)(hidden / 8)), (int)(hidden / 8), lanes_per_row, chunks_per_lane);
     return GPUK_OK;
 }
 

@@ -40,6 +40,11 @@ extern "C" int gpuk_set_tuning(const char *key, int value) {
         gpuk::set_norm_quant_tuning(6, value);
         return GPUK_OK;
     }
+    if (strcmp(key, "norm_quant_launches") == 0) {  // 0 = built-in rule, 1 = always one, 2 = two wherever each half fits a round
+        if (value < 0 || value > 2) return GPUK_ERR_INVALID_ARG;
+        gpuk::set_norm_quant_tuning(7, value);
+        return GPUK_OK;
+    }
     if (strcmp(key, "rope_unit_gate") == 0) {
         if (value < -1 || value > 5000) return GPUK_ERR_INVALID_ARG;
         gpuk::set_rope_tuning(6, value);

@@ -192,7 +192,7 @@ int gpuk_add_rmsnorm_quant_traffic_only(const void *x, const void *residual_in, 
 /*
  * The launch shape gpuk_add_rmsnorm_quant picks for a batch: lanes per token row (= workgroup size; one workgroup
  * per row) and chunks per lane (8 elements of a 16-bit type, 4 of fp32 / fp64; 0: rows too long for registers, swept
- * three times).  For reports.
+ * three times); of a batch that runs as two launches, the first one's.  For reports.
  */
 int gpuk_add_rmsnorm_quant_launch_shape(int64_t tokens, int64_t hidden, int dtype, int *lanes_per_row,
                                         int *chunks_per_lane);
@@ -222,6 +222,8 @@ int gpuk_increment_floats(float *data, int64_t n, void *stream);
  * per row), "norm_quant_row_group_shift" (log2 of the run of consecutive rows one XCD takes; -1, not 0, restores the
  * built-in rule), "norm_quant_gate" (how long, in ticks of 10 ns after a wave's entry, the stores of the norm-quant
  * kernel are held back so that the reads of a batch the chip holds at once go first: -1 the built-in rule, 0 never),
+ * "norm_quant_launches" (1: a call is always one launch; 2: two, of half the rows each, wherever the batch is more
+ * than one round of workgroups and at most two),
  * "rope_block_threads" (64/128/256/512 lanes per workgroup of the rope kernel), "rope_stream_rows" (output rows of
  * the rope kernels stored past the L2: 1 never, 2 always), "rope_merge_rows" (1: never let the lanes of an mRoPE
  * token load their cos/sin pieces straight from the row of their axis), "rope_token_waves" (the kernel in which one

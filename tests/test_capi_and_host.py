@@ -74,6 +74,7 @@ def test_argument_validation_needs_no_gpu():
     assert L.gpuk_empty_grid(4, 256, 1 << 20, None) == 1 and L.gpuk_empty_grid(0, 256, 0, None) == 0
     assert L.gpuk_set_tuning(b"no_such_knob", 1) == 1 and L.gpuk_set_tuning(b"norm_quant_nchunk", 3) == 1
     assert L.gpuk_set_tuning(b"norm_quant_nchunk", 0) == 0
+    assert L.gpuk_set_tuning(b"norm_quant_launches", 3) == 1 and L.gpuk_set_tuning(b"norm_quant_launches", 0) == 0
 
 
 def test_torch_library_registers_reference_schemas():
@@ -266,6 +267,14 @@ def test_launch_shape_report():
     assert capi.add_rmsnorm_quant_launch_shape(1025, 7168) == (256, 4)
     assert capi.add_rmsnorm_quant_launch_shape(2048, 8192) == (256, 4)
     assert capi.add_rmsnorm_quant_launch_shape(2049, 8192) == (512, 2)
+    # from 1.1 rounds to two the call is two launches; the report is the first one's (1280 of 2600 rows, 1536 of 3000)
+    assert capi.add_rmsnorm_quant_launch_shape(2252, 8192) == (512, 2)
+    assert capi.add_rmsnorm_quant_launch_shape(2600, 8192) == (256, 4)
+    assert capi.add_rmsnorm_quant_launch_shape(3000, 7168) == (256, 4)
+    assert capi.add_rmsnorm_quant_launch_shape(4097, 7168) == (448, 2)
+    # workgroups of five waves: a compute unit takes five of them, not six
+    assert capi.add_rmsnorm_quant_launch_shape(1280, 5120) == (320, 2)
+    assert capi.add_rmsnorm_quant_launch_shape(1281, 5120) == (192, 4)
     assert capi.add_rmsnorm_quant_launch_shape(1, 4096) == (256, 2)
     lanes, chunks = capi.add_rmsnorm_quant_launch_shape(4, 65600 * 2)    # rows that do not stay in registers
     assert chunks == 0 and lanes % 64 == 0

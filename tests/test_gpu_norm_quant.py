@@ -61,7 +61,12 @@ def check(inp, quant, got, fp8_max=448.0, static_scale=None, tag=""):
             else:
                 assert_codes_close(norm, norm_ref, f"{tag} fp8 codes")
                 if quant == 1:
-                    assert_scales_close(scale, scale_ref, f"{tag} scale_out")
+                    # (rows whose scale is further off are held, below, to the oracle at a moved rstd, bit for bit:
+                    # the row's largest value sat on a rounding tie of the 16-bit type and rstd's last bit decided it)
+                    s_got, s_want = scale.cpu().flatten().double(), scale_ref.flatten().double()
+                    scale_moved = ((s_got - s_want).abs() > 1e-6 * s_want.abs()) | (s_got.isnan() != s_want.isnan())
+                    assert_scales_close(scale.cpu().flatten()[~scale_moved], scale_ref.flatten()[~scale_moved], f"{tag} scale_out")
+                    assert int(scale_moved.sum()) <= max(1, rows // 1000), f"{tag}: {int(scale_moved.sum())} rows with a scale beyond 1e-6"
             exact = (g_norm == raw(norm_ref)).float().mean().item() if rows else 1.0
         explained |= same
         if abs(off) <= 1:
@@ -233,6 +238,41 @@ def test_batches_between_one_and_two_rounds(device, tokens, hidden, dtype):
     for quant in (0, 1, 3):
         st = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
         check(inp, quant, run_capi(inp, quant, device, static_scale=st), static_scale=st, tag=f"[{tokens}x{hidden} q{quant}]")
+
+
+@pytest.mark.parametrize("tokens,hidden,dtype", [(2300, 7168, torch.bfloat16), (4096, 8192, torch.bfloat16),
+                                                 (4600, 4096, torch.bfloat16), (1500, 10240, torch.bfloat16),
+                                                 (2900, 5120, torch.float16), (9300, 1024, torch.bfloat16)])
+def test_batches_of_one_to_two_rounds_take_two_launches(device, tokens, hidden, dtype):
+    """From 1.1 rounds of workgroups to two a call is two launches of about half the rows each (the first a whole
+    number of rows per compute unit), each one round with the store gate.  The oracle's bits in every quant mode, as
+    for one launch over the whole batch (whose lanes sum a row's squares in another order, so the two are each held to
+    the oracle, not to each other, beyond the residual); the same bits with the residual stream in place."""
+    from gpuk_amd import capi
+
+    inp = workloads.norm_quant_inputs(tokens, hidden, seed=tokens + 3, res_sigma=2.0, outlier_frac=0.01, dtype=dtype)
+    for quant in (0, 1, 3):
+        print(f"case two launches {tokens}x{hidden} {dtype} quant={quant}", flush=True)
+        st = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
+        two = run_capi(inp, quant, device, static_scale=st)
+        check(inp, quant, two, static_scale=st, tag=f"[two launches {tokens}x{hidden} q{quant}]")
+        capi.set_tuning("norm_quant_launches", 1)
+        try:
+            one = run_capi(inp, quant, device, static_scale=st)
+        finally:
+            capi.set_tuning("norm_quant_launches", 0)
+        check(inp, quant, one, static_scale=st, tag=f"[one launch {tokens}x{hidden} q{quant}]")
+        assert_bits_equal(two[0], one[0], "residual_out, two launches against one")
+        # in place: residual_out is residual_in
+        x, r, g = inp.x.to(device), inp.residual.to(device), inp.gamma.to(device)
+        norm = torch.empty_like(two[1])
+        scale = None if quant == 0 else (torch.empty((tokens, 1), dtype=torch.float32, device=device) if quant == 1 else st.to(device).float().reshape(1))
+        capi.add_rmsnorm_quant(x, r, g, r, norm, scale, inp.eps, quant)
+        torch.cuda.synchronize()
+        assert_bits_equal(r, two[0], "residual stream in place")
+        assert_bits_equal(norm, two[1], "norm_out with the residual stream in place")
+        if quant == 1:
+            assert_bits_equal(scale, two[2], "scales with the residual stream in place")
 
 
 @pytest.mark.parametrize("alias", ["residual_in", "x"])
