@@ -106,13 +106,14 @@ def test_compiled_function_keeps_the_writes(device):
     assert_scales_close(traced[2], scale_ref, "compiled scales")
 
 
-def test_env_capture_replays(device):
+@pytest.mark.parametrize("tokens,hidden", [(32, 7168), (2048, 7168), (2600, 8192)])
+def test_env_capture_replays(device, tokens, hidden):
     """GPUKDistEnv.capture() around a HIP graph capture of the fused call: every replay, with fresh inputs copied
-    into the captured buffers and eager work in between, equals the eager result on the same inputs."""
+    into the captured buffers and eager work in between, equals the eager result on the same inputs.  (32 rows: one
+    ungated launch; 2048: one round of gated workgroups; 2600 x 8192: two gated launches recorded for the one call.)"""
     import gpuk_amd
 
     env = gpuk_amd.GPUKDistEnv(device_id=device.index or 0)
-    tokens, hidden = 32, 7168
     static_x = torch.zeros((tokens, hidden), dtype=torch.bfloat16, device=device)
     static_r = torch.zeros_like(static_x)
     gamma = (1 + 0.1 * torch.randn(hidden, device=device)).bfloat16()
