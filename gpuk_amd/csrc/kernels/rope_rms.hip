@@ -654,7 +654,23 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t w = blockIdx.x * 4 + wave;
     if (w >= num_waves) return;
-    const uint32_t t = w, t2 = w + num_waves;  // the wave's token(s)
+    // The wave's token(s).  TWO: the tokens beyond num_waves (a multiple of 1024 wherever there are any: a whole
+    // number of waves on every SIMD) ride as second tokens, dealt out evenly over the compute units -- workgroup g runs
+    // on compute unit g mod 256 while the launch is one round, so the waves of a compute unit are w = 4 (cu + 256 l) + i,
+    // ranked l, i here, and the first extra / 256 of each rank order take one (the remainder: one more on the first units).
+    // (Any other num_waves: wave w takes token w + num_waves as well, where there is one.)
+    const uint32_t t = w;
+    uint32_t t2 = num_tokens;
+    if constexpr (TWO) {
+        if (num_waves & 1023u) {
+            t2 = w + num_waves;
+        } else {
+            const uint32_t extra = num_tokens - num_waves, each = extra >> 8, more = extra & 255u;
+            const uint32_t cu = (w >> 2) & 255u, rank = ((w >> 10) << 2) | (w & 3u);
+            if (rank < each) t2 = num_waves + cu * each + rank;
+            else if (rank == each && cu < more) t2 = num_waves + (each << 8) + cu;
+        }
+    }
     const bool second = TWO && t2 < num_tokens;  // wave-uniform
     const int lane = threadIdx.x & 63, sub = lane % LPH, hl = lane / LPH;
     const int heads_qk = hq + hk, heads_all = heads_qk + hv, v_chunks = hv * (D / 8);
@@ -1160,21 +1176,23 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     // 32+8+8 heads, 9.1 against 9.5 at 2100 tokens of 28+4+4; from there on this one is: 32+8+8 heads 10.3 against
     // 11.1 us at 2048 tokens, 13.6 against 14.8 at 3000, 16.6 against 17.3 at 3700, 16.2 against 18.2 at 4096; 28+4+4
     // heads with three axes 10.0 against 11.7 us at 3000 tokens, 12.2 against 14.5 at 4096).
-    // With two tokens per wave only where the waves fill the SIMDs evenly, three or four on each: 19.1 against 20.3 us
-    // at 6144 tokens of 28+4+4 heads, 24.0 against 25.8 at 8192, but 22.8 against 23.1 at 7168 (three and a half
-    // waves per SIMD: the fuller ones set the time) and 17.9 against 17.5 at 5120.
+    // With two tokens per wave from there to twice that many tokens: 4096 waves, four on every SIMD, one token each and
+    // the others dealt out evenly.  The SIMD with the most tokens sets the time (the rotation arithmetic of its waves
+    // is two thirds of the launch), so the time goes up in steps of 1024 tokens where the kernel above is linear; this
+    // one is ahead or level everywhere (graph replays, 28+4+4 heads, one axis / three: 16.1 / 16.4 against 17.2 / 17.5 us
+    // at 4800 tokens, 18.2 / 18.5 against 18.4 / 18.8 at 5200, 19.1 / 19.6 against 21.1 / 21.5 at 6144, 21.7 / 21.7 against
+    // 23.5 / 23.7 at 7000, 25.0 / 24.4 against 24.9 / 25.3 at 7500, 25.8 / 25.6 against 26.6 / 27.1 at 8192; 15.1 / 15.8
+    // against 15.3 / 15.5 at 4100).  Half as many waves with two tokens each were behind that: 20.0 at 6144 tokens.
     // (in place, with no V row and no scatter, the kernel above holds out a little longer: 9.0 against 9.5 us at 2048
     // tokens of 32+8 heads, then 11.9 against 11.2 at 3000, 15.4 against 13.7 at 4096; 28+4 heads with three axes 10.7
     // against 9.5 at 3000 tokens, 13.2 against 11.5 at 4096, 18.4 against 17.4 at 6144 and 23.2 against 21.6 at 8192 with
     // two tokens per wave)
     const bool large = a.total_units >= (set_kv ? kResidentUnits + kResidentUnits / 4 : kResidentUnits + 2 * kResidentUnits / 5);
-    const uint32_t waves2 = (a.num_tokens + 1) / 2, rounds2 = (waves2 + 1023) / 1024;
-    const bool even2 = rounds2 >= 3 && 100 * (uint64_t)waves2 >= 94 * (uint64_t)rounds2 * 1024;
     // (with an fp8 cache the conversions lengthen the wave and the gate hardly matters; one token per wave is still
     // ahead once the batch is large: 28+4+4 heads 10.8 against 11.9 us at 3000 tokens, 13.3 against 14.2 at 4096; 32+8+8
     // heads 16.8 against 17.6 at 4096, level at 3000, behind at 2560)
     const bool large_fp8 = a.total_units >= (a.units_per_token == 4 ? kResidentUnits + kResidentUnits / 4 : 7 * kResidentUnits / 4);
-    const bool by_rule = g_token_waves == 0 && (two ? even2 : (kv_fp8 ? large_fp8 : large));
+    const bool by_rule = g_token_waves == 0 && (two || (kv_fp8 ? large_fp8 : large));
     p.token_waves = (one || two) && (g_token_waves >= 2 || by_rule);
     p.two_tokens = p.token_waves && two;
     // (with two tokens per wave the full read time: 24.4 us at 8192 tokens of 28+4+4 heads with three axes, against 25.4
@@ -1217,7 +1235,9 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     p.blocks = (a.total_units + units_per_block - 1) / units_per_block;
     if (p.token_waves) {
         p.threads = 256;
-        p.token_wave_count = p.two_tokens ? (a.num_tokens + 1) / 2 : a.num_tokens;
+        // (two tokens per wave: every SIMD's four waves take one token each and the rest are dealt out over them; a
+        // batch that two tokens per wave are forced onto although one would do is halved instead)
+        p.token_wave_count = !p.two_tokens ? a.num_tokens : a.num_tokens > kTokenWaveCapacity ? kTokenWaveCapacity : (a.num_tokens + 1) / 2;
         p.blocks = (p.token_wave_count + 3) / 4;
         p.stream = true;
     }

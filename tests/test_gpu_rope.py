@@ -445,28 +445,61 @@ def test_token_kernel_random_shapes(device, seed):
     check_inplace(inp, got_inplace, f"[token fuzz {seed}, in place]")
 
 
+@pytest.mark.parametrize("tokens", [4097, 4351, 4352, 4608, 5121, 6143, 7424, 8191, 8192])
+def test_second_tokens_are_dealt_out_over_every_wave(device, tokens):
+    """Between 4097 and 8192 tokens the kernel runs 4096 waves; wave 4 (cu + 256 l) + i takes, beside token w, one of
+    the tokens from 4096 on according to its place (l, i) among the waves of compute unit cu.  Every token must be
+    taken exactly once: the same bits as the kernel with one wave per group of heads, q_out and both caches (tokens
+    without a slot among them), with three axes and in place as well."""
+    from gpuk_amd import capi
+
+    for mrope in (False, True):
+        print(f"case second tokens T={tokens} mrope={mrope}", flush=True)
+        inp = make(tokens, 24, 128, True, seed=tokens, mrope=mrope, hk=8, hv=3)
+        if mrope:
+            inp.mrope_section = [16, 24, 24]
+        inp.kv_loc[5::11] = -1
+        n_axes = 3 if mrope else 1
+        assert capi.rope_rms_launch_shape(tokens, 24, 8, 3, 128, n_axes, inp.qkv.dtype, True, False) == (1024, 256, True, 2)
+        got, got_inplace = run_set_kv(inp, device), run_inplace(inp, device)
+        try:
+            capi.set_tuning("rope_token_waves", 1)
+            base, base_inplace = run_set_kv(inp, device), run_inplace(inp, device)
+        finally:
+            capi.set_tuning("rope_token_waves", 0)
+        raw = lambda t: t.cpu().contiguous().view(torch.uint8)
+        for name, x, y in zip(("q_out", "k_cache", "v_cache"), got[:3], base[:3]):
+            assert torch.equal(raw(x), raw(y)), f"{name}: the two kernels differ"
+        assert torch.equal(raw(got_inplace), raw(base_inplace)), "in place: the two kernels differ"
+    check_set_kv(inp, got, f"[second tokens T={tokens}]")
+
+
 def test_one_wave_per_token_kernel_by_rule(device):
     """The launcher's rule takes that kernel where the other one is clearly past what it holds at once (from 10240
-    groups of heads: 2560 tokens of 28+4 heads, not 2559) up to the 4096 tokens it holds itself; with two tokens per
-    wave where those waves fill the SIMDs evenly (6144 and 8192 tokens here, not 4097, 5000 or 8193); with one or three
-    position axes; with an fp8 cache one token per wave only.  Every choice meets the oracle."""
+    groups of heads: 2560 tokens of 28+4+4 heads, not 2559) up to the 4096 tokens it holds itself, and from there to
+    8192 tokens with 4096 waves that take one token each and share out the rest (4097, 5000, 7169, 8192 tokens here,
+    not 8193); with one or three position axes; with an fp8 cache one token per wave only.  Every choice meets the
+    oracle."""
     from gpuk_amd import capi
 
     for tokens, mrope, fp8, expect in ((2559, False, False, 0), (2560, False, False, 1), (3500, True, False, 1),
-                                       (4096, False, False, 1), (4097, False, False, 0), (5000, True, False, 0),
-                                       (6144, True, False, 2), (8192, True, False, 2), (8192, False, False, 2),
-                                       (8193, False, False, 0), (2500, False, True, 0), (4000, False, True, 1), (6144, False, True, 0)):
+                                       (4096, False, False, 1), (4097, False, False, 2), (5000, True, False, 2),
+                                       (6144, True, False, 2), (7169, False, False, 2), (8192, True, False, 2),
+                                       (8192, False, False, 2), (8193, False, False, 0), (2500, False, True, 0),
+                                       (4000, False, True, 1), (6144, False, True, 0)):
         groups, lanes, _, token_waves = capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 3 if mrope else 1, torch.bfloat16, True, fp8)
-        waves = (tokens + 1) // 2 if expect == 2 else tokens
+        waves = 4096 if expect == 2 else tokens
         assert token_waves == expect and (not expect or (groups, lanes) == ((waves + 3) // 4, 256)), (tokens, fp8, groups, lanes)
         inp = make(tokens, 28, 128, True, seed=tokens + 1, mrope=mrope, fp8=fp8, hk=4, hv=4)
         if mrope:
             inp.mrope_section = [16, 24, 24]
+        if expect == 2:
+            inp.kv_loc[::7] = -1   # tokens without a slot among the first and the second tokens of the waves
         check_set_kv(inp, run_set_kv(inp, device), f"[rule T={tokens} mrope={mrope} fp8={fp8}]")
     # 32+8+8 heads: five groups per token, one token per wave only
     assert capi.rope_rms_launch_shape(4097, 32, 8, 8, 128)[3] == 0
     # in place the other kernel holds out a little longer (to 11468 groups of heads)
-    for tokens, mrope, expect in ((2800, False, 0), (3000, True, 1), (8192, True, 2)):
+    for tokens, mrope, expect in ((2800, False, 0), (3000, True, 1), (4500, False, 2), (7800, True, 2), (8192, True, 2)):
         assert capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 3 if mrope else 1, torch.bfloat16, False, False)[3] == expect
         inp = make(tokens, 28, 128, True, seed=tokens + 2, mrope=mrope, hk=4, hv=4)
         if mrope:
