@@ -445,12 +445,13 @@ def test_token_kernel_random_shapes(device, seed):
     check_inplace(inp, got_inplace, f"[token fuzz {seed}, in place]")
 
 
-@pytest.mark.parametrize("tokens", [4097, 4351, 4352, 4608, 5121, 6143, 7424, 8191, 8192])
+@pytest.mark.parametrize("tokens", [2047, 2048, 4096, 4097, 4351, 4352, 4608, 5121, 6143, 7424, 8191, 8192])
 def test_second_tokens_are_dealt_out_over_every_wave(device, tokens):
     """Between 4097 and 8192 tokens the kernel runs 4096 waves; wave 4 (cu + 256 l) + i takes, beside token w, one of
     the tokens from 4096 on according to its place (l, i) among the waves of compute unit cu.  Every token must be
     taken exactly once: the same bits as the kernel with one wave per group of heads, q_out and both caches (tokens
-    without a slot among them), with three axes and in place as well."""
+    without a slot among them), with three axes and in place as well.  (Up to 4096 tokens the arrangement is forced:
+    half as many waves, which deal in the same way where they come to a multiple of 1024.)"""
     from gpuk_amd import capi
 
     for mrope in (False, True):
@@ -460,9 +461,11 @@ def test_second_tokens_are_dealt_out_over_every_wave(device, tokens):
             inp.mrope_section = [16, 24, 24]
         inp.kv_loc[5::11] = -1
         n_axes = 3 if mrope else 1
-        assert capi.rope_rms_launch_shape(tokens, 24, 8, 3, 128, n_axes, inp.qkv.dtype, True, False) == (1024, 256, True, 2)
-        got, got_inplace = run_set_kv(inp, device), run_inplace(inp, device)
         try:
+            capi.set_tuning("rope_token_waves", 0 if tokens > 4096 else 3)
+            waves = 4096 if tokens > 4096 else (tokens + 1) // 2
+            assert capi.rope_rms_launch_shape(tokens, 24, 8, 3, 128, n_axes, inp.qkv.dtype, True, False) == ((waves + 3) // 4, 256, True, 2)
+            got, got_inplace = run_set_kv(inp, device), run_inplace(inp, device)
             capi.set_tuning("rope_token_waves", 1)
             base, base_inplace = run_set_kv(inp, device), run_inplace(inp, device)
         finally:
