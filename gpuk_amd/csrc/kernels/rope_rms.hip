@@ -666,8 +666,10 @@ rope_rms_token_kernel(const void *qkv_in, const int64_t *positions, uint32_t num
             t2 = w + num_waves;
         } else {
             const uint32_t extra = num_tokens - num_waves, each = extra >> 8, more = extra & 255u;
-            const uint32_t cu = (w >> 2) & 255u, rank = ((w >> 10) << 2) | (w & 3u);
-            if (rank < each) t2 = num_waves + cu * each + rank;
+            const uint32_t cu = (w >> 2) & 255u, layer = w >> 10, rank = (layer << 2) | (w & 3u);
+            // (in wave order as far as whole layers of 1024 waves go -- neighbouring workgroups then take neighbouring
+            // tokens, 1 % at 8192 tokens -- then the waves of the part layer, then the remainder)
+            if (rank < each) t2 = num_waves + (layer < (each >> 2) ? w : (layer << 10) + cu * (each & 3u) + (w & 3u));
             else if (rank == each && cu < more) t2 = num_waves + (each << 8) + cu;
         }
     }
@@ -1181,8 +1183,8 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     // is two thirds of the launch), so the time goes up in steps of 1024 tokens where the kernel above is linear; this
     // one is ahead or level everywhere (graph replays, 28+4+4 heads, one axis / three: 16.1 / 16.4 against 17.2 / 17.5 us
     // at 4800 tokens, 18.2 / 18.5 against 18.4 / 18.8 at 5200, 19.1 / 19.6 against 21.1 / 21.5 at 6144, 21.7 / 21.7 against
-    // 23.5 / 23.7 at 7000, 25.0 / 24.4 against 24.9 / 25.3 at 7500, 25.8 / 25.6 against 26.6 / 27.1 at 8192; 15.1 / 15.8
-    // against 15.3 / 15.5 at 4100).  Half as many waves with two tokens each were behind that: 20.0 at 6144 tokens.
+    // 23.5 / 23.7 at 7000, 24.2 / 24.4 against 24.7 / 25.3 at 7500, 25.3 / 25.3 against 26.8 / 27.3 at 8192; level below
+    // 4608 tokens, where the kernel above stays).  Half as many waves with two tokens each were behind that: 20.0 at 6144 tokens.
     // (in place, with no V row and no scatter, the kernel above holds out a little longer: 9.0 against 9.5 us at 2048
     // tokens of 32+8 heads, then 11.9 against 11.2 at 3000, 15.4 against 13.7 at 4096; 28+4 heads with three axes 10.7
     // against 9.5 at 3000 tokens, 13.2 against 11.5 at 4096, 18.4 against 17.4 at 6144 and 23.2 against 21.6 at 8192 with
@@ -1192,7 +1194,8 @@ RopePlan plan_rope(const RopeArgs &a, int D, int axes, bool set_kv, bool kv_fp8)
     // ahead once the batch is large: 28+4+4 heads 10.8 against 11.9 us at 3000 tokens, 13.3 against 14.2 at 4096; 32+8+8
     // heads 16.8 against 17.6 at 4096, level at 3000, behind at 2560)
     const bool large_fp8 = a.total_units >= (a.units_per_token == 4 ? kResidentUnits + kResidentUnits / 4 : 7 * kResidentUnits / 4);
-    const bool by_rule = g_token_waves == 0 && (two || (kv_fp8 ? large_fp8 : large));
+    const bool extra_enough = a.num_tokens >= kTokenWaveCapacity + kTokenWaveCapacity / 8;  // (level or 1 % behind below: 15.4 against 15.2 us at 4100 tokens)
+    const bool by_rule = g_token_waves == 0 && (two ? extra_enough : (kv_fp8 ? large_fp8 : large));
     p.token_waves = (one || two) && (g_token_waves >= 2 || by_rule);
     p.two_tokens = p.token_waves && two;
     // (with two tokens per wave the full read time: 24.4 us at 8192 tokens of 28+4+4 heads with three axes, against 25.4

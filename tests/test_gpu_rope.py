@@ -450,8 +450,8 @@ def test_second_tokens_are_dealt_out_over_every_wave(device, tokens):
     """Between 4097 and 8192 tokens the kernel runs 4096 waves; wave 4 (cu + 256 l) + i takes, beside token w, one of
     the tokens from 4096 on according to its place (l, i) among the waves of compute unit cu.  Every token must be
     taken exactly once: the same bits as the kernel with one wave per group of heads, q_out and both caches (tokens
-    without a slot among them), with three axes and in place as well.  (Up to 4096 tokens the arrangement is forced:
-    half as many waves, which deal in the same way where they come to a multiple of 1024.)"""
+    without a slot among them), with three axes and in place as well.  (Below 4608 tokens the arrangement is forced;
+    up to 4096 tokens that is half as many waves, which deal in the same way where they come to a multiple of 1024.)"""
     from gpuk_amd import capi
 
     for mrope in (False, True):
@@ -462,7 +462,7 @@ def test_second_tokens_are_dealt_out_over_every_wave(device, tokens):
         inp.kv_loc[5::11] = -1
         n_axes = 3 if mrope else 1
         try:
-            capi.set_tuning("rope_token_waves", 0 if tokens > 4096 else 3)
+            capi.set_tuning("rope_token_waves", 0 if tokens >= 4608 else 3)
             waves = 4096 if tokens > 4096 else (tokens + 1) // 2
             assert capi.rope_rms_launch_shape(tokens, 24, 8, 3, 128, n_axes, inp.qkv.dtype, True, False) == ((waves + 3) // 4, 256, True, 2)
             got, got_inplace = run_set_kv(inp, device), run_inplace(inp, device)
@@ -480,13 +480,13 @@ def test_second_tokens_are_dealt_out_over_every_wave(device, tokens):
 def test_one_wave_per_token_kernel_by_rule(device):
     """The launcher's rule takes that kernel where the other one is clearly past what it holds at once (from 10240
     groups of heads: 2560 tokens of 28+4+4 heads, not 2559) up to the 4096 tokens it holds itself, and from there to
-    8192 tokens with 4096 waves that take one token each and share out the rest (4097, 5000, 7169, 8192 tokens here,
-    not 8193); with one or three position axes; with an fp8 cache one token per wave only.  Every choice meets the
-    oracle."""
+    8192 tokens, once an eighth of them have a second token, with 4096 waves that take one token each and share out
+    the rest (4608, 5000, 7169, 8192 tokens here, not 4607 or 8193); with one or three position axes; with an fp8
+    cache one token per wave only.  Every choice meets the oracle."""
     from gpuk_amd import capi
 
     for tokens, mrope, fp8, expect in ((2559, False, False, 0), (2560, False, False, 1), (3500, True, False, 1),
-                                       (4096, False, False, 1), (4097, False, False, 2), (5000, True, False, 2),
+                                       (4096, False, False, 1), (4607, False, False, 0), (4608, False, False, 2), (5000, True, False, 2),
                                        (6144, True, False, 2), (7169, False, False, 2), (8192, True, False, 2),
                                        (8192, False, False, 2), (8193, False, False, 0), (2500, False, True, 0),
                                        (4000, False, True, 1), (6144, False, True, 0)):
@@ -502,7 +502,7 @@ def test_one_wave_per_token_kernel_by_rule(device):
     # 32+8+8 heads: five groups per token, one token per wave only
     assert capi.rope_rms_launch_shape(4097, 32, 8, 8, 128)[3] == 0
     # in place the other kernel holds out a little longer (to 11468 groups of heads)
-    for tokens, mrope, expect in ((2800, False, 0), (3000, True, 1), (4500, False, 2), (7800, True, 2), (8192, True, 2)):
+    for tokens, mrope, expect in ((2800, False, 0), (3000, True, 1), (4500, False, 0), (4700, False, 2), (7800, True, 2), (8192, True, 2)):
         assert capi.rope_rms_launch_shape(tokens, 28, 4, 4, 128, 3 if mrope else 1, torch.bfloat16, False, False)[3] == expect
         inp = make(tokens, 28, 128, True, seed=tokens + 2, mrope=mrope, hk=4, hv=4)
         if mrope:
