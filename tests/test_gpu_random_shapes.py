@@ -36,6 +36,32 @@ def test_norm_quant_random_shapes(device, tokens, hidden, quant, dtype):
                      tag=f"[{tokens}x{hidden} q{quant}]")
 
 
+def norm_quant_round_cases(n=14):
+    """Batches of a fifth of a round of workgroups to two and a half: the store gate, four chunks per lane, two
+    launches per call and plain several-round launches, whichever the launcher's rules pick."""
+    rng = random.Random(4242)
+    cases = []
+    for i in range(n):
+        hidden = 8 * rng.choice([128, 256, 320, 384, 512, 640, 768, 896, 1024, 1280, 2048])
+        waves4 = -(-(hidden // 8) // 4 // 64)                # waves per row at four chunks per lane
+        round_rows = 256 * (32 // waves4)
+        tokens = max(1, min(int(round_rows * rng.uniform(0.2, 2.5)), 20_000_000 // hidden))
+        cases.append((tokens, hidden, rng.choice([0, 1, 3]), rng.choice([torch.bfloat16, torch.float16])))
+    return cases
+
+
+@pytest.mark.parametrize("tokens,hidden,quant,dtype", norm_quant_round_cases())
+def test_norm_quant_random_batches_around_a_round(device, tokens, hidden, quant, dtype):
+    from gpuk_amd import capi
+
+    print(f"case random norm-quant around a round tokens={tokens} hidden={hidden} quant={quant} dtype={dtype} "
+          f"shape={capi.add_rmsnorm_quant_launch_shape(tokens, hidden, dtype)}", flush=True)
+    inp = workloads.norm_quant_inputs(tokens, hidden, seed=tokens * 13 + hidden, res_sigma=1.5, outlier_frac=0.01, dtype=dtype)
+    static = O.static_scale_for(inp.x, inp.residual, inp.gamma, inp.eps) if quant == 3 else None
+    check_norm_quant(inp, quant, run_norm_quant(inp, quant, device, static_scale=static), static_scale=static,
+                     tag=f"[{tokens}x{hidden} q{quant}]")
+
+
 def rope_cases(n=36):
     rng = random.Random(77)
     cases = []
